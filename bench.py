@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the optimizer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A "step" is one pass of the fused AdamW kernel over every tensor of the
+workload, with all operands already resident in HBM.  The default workload is
+BASELINE config 1: stochastic_rounding mode over the Llama-style 1.1B
+parameter set (201 tensors, 1,100,048,384 elements, 14 algorithmic bytes per
+element).  Prints ONE JSON line.
+
+Only one GPU is used; ``--gpus N`` with N > 1 exits with a message.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+BYTES_PER_ELEM = {
+    "stochastic_rounding": 14,
+    "fp32_master": 20,
+    "fp31_master": 18,
+    "fp32_master_custom_rounding": 18,
+}
+
+
+def llama_shapes(hidden, inter, layers, q_heads, kv_heads, head_dim, vocab):
+    """Parameter shapes of an untied Llama-style decoder, in module order."""
+    shapes = [("embed_tokens", (vocab, hidden))]
+    for i in range(layers):
+        shapes += [
+            (f"l{i}.input_norm", (hidden,)),
+            (f"l{i}.q_proj", (q_heads * head_dim, hidden)),
+            (f"l{i}.k_proj", (kv_heads * head_dim, hidden)),
+            (f"l{i}.v_proj", (kv_heads * head_dim, hidden)),
+            (f"l{i}.o_proj", (hidden, q_heads * head_dim)),
+            (f"l{i}.post_norm", (hidden,)),
+            (f"l{i}.gate_proj", (inter, hidden)),
+            (f"l{i}.up_proj", (inter, hidden)),
+            (f"l{i}.down_proj", (hidden, inter)),
+        ]
+    shapes += [("final_norm", (hidden,)), ("lm_head", (vocab, hidden))]
+    return shapes
+
+
+WORKLOADS = {
+    # BASELINE config 1
+    "c1_sr_llama1b": dict(
+        mode="stochastic_rounding",
+        shapes=llama_shapes(2048, 5632, 22, 32, 4, 64, 32000),
+        clip=False,
+    ),
+    # BASELINE config 0 (one flat tensor)
+    "c0_fp32_master_16m": dict(mode="fp32_master", shapes=[("flat", (16_777_216,))], clip=False),
+    # BASELINE config 2 kernel leg: fp31_master + fused clip on Llama-3-8B shapes
+    "c2_fp31_clip_llama8b": dict(
+        mode="fp31_master",
+        shapes=llama_shapes(4096, 14336, 32, 32, 8, 128, 128256),
+        clip=True,
+    ),
+}
+
+
+def numel(shape):
+    n = 1
+    for s in shape:
+        n *= s
+    return n
+
+
+def make_tensors(mode, shapes, device, seed=0):
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    out = []
+    for _, shape in shapes:
+        n = numel(shape)
+        p = (torch.randn(n, device=device, generator=g) * 0.02).to(torch.bfloat16)
+        st = {
+            "grad": (torch.randn(n, device=device, generator=g) * 1e-3).to(torch.bfloat16),
+            "exp_avg": (torch.randn(n, device=device, generator=g) * 1e-4).to(torch.bfloat16),
+            "exp_avg_sq": ((torch.randn(n, device=device, generator=g) * 1e-3) ** 2).to(
+                torch.bfloat16
+            ),
+        }
+        if mode == "fp32_master":
+            st["master_params"] = p.float()
+        elif mode in ("fp31_master", "fp32_master_custom_rounding"):
+            st["rounding_error"] = torch.zeros(n, dtype=torch.int16, device=device)
+        out.append((p, st))
+    return out
+
+
+def cpu_baseline(mode, target_elems=32 * 1024 * 1024, iters=3):
+    """The same update math in PyTorch eager on this host's cores, on a bounded
+    sample of the workload (one flat tensor of ``target_elems`` elements)."""
+    import torch
+
+    from oracle import folded_betas, torch_eager
+
+    n = target_elems
+    g = torch.Generator().manual_seed(0)
+    p = (torch.randn(n, generator=g) * 0.02).to(torch.bfloat16)
+    st = {
+        "grad": (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16),
+        "exp_avg": (torch.randn(n, generator=g) * 1e-4).to(torch.bfloat16),
+        "exp_avg_sq": ((torch.randn(n, generator=g) * 1e-3) ** 2).to(torch.bfloat16),
+    }
+    b1h, b2h = folded_betas(0.9, 0.999, 10)
+    args = (1e-4, 0.01, b1h, b2h, 1e-8, True)
+    if mode == "stochastic_rounding":
+        def run():
+            r = torch.randint(0, 65536, (n,), dtype=torch.int32)
+            torch_eager.adam_step_stochastic_rounding(p, st, *args, r)
+    elif mode == "fp32_master":
+        st["master_params"] = p.float()
+        def run():
+            torch_eager.adam_step_fp32_master(p, st, *args)
+    else:
+        st["rounding_error"] = torch.zeros(n, dtype=torch.int16)
+        fn = (torch_eager.adam_step_fp31_master if mode == "fp31_master"
+              else torch_eager.adam_step_custom_rounding)
+        def run():
+            fn(p, st, *args)
+    run()  # warm-up
+    times = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    best = sorted(times)[len(times) // 2]
+    return {
+        "value": round(n * BYTES_PER_ELEM[mode] / best / 1e9, 3),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"one flat tensor of {n} elements, {mode}, torch eager fp32 on CPU, "
+                  f"median of {iters} passes ({best:.3f} s per pass)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c1_sr_llama1b", choices=sorted(WORKLOADS))
+    ap.add_argument("--rng", default=None, choices=[None, "triton", "x8"],
+                    help="stochastic_rounding bit layout (default: the optimizer's own, x8)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-events", action="store_true",
+                    help="skip per-launch HIP events (used for profiler runs)")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (no collectives, no sharding); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from offload_adam_amd import _lib, kernels
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _lib.load()  # fails loudly when the HIP library is not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    wl = WORKLOADS[args.workload]
+    mode = wl["mode"]
+    tensors = make_tensors(mode, wl["shapes"], dev)
+    step_fn = getattr(kernels, "adam_step_" + mode)
+    clip = torch.tensor(0.3359375, dtype=torch.bfloat16, device=dev) if wl["clip"] else None
+    total_elems = sum(p.numel() for p, _ in tensors)
+    bytes_per_step = total_elems * BYTES_PER_ELEM[mode]
+    kw = {}
+    if mode == "stochastic_rounding" and args.rng is not None:
+        kw["rng"] = args.rng
+        kw["seed"] = 1
+
+    def one_step(step_no, events=None):
+        for i, (p, st) in enumerate(tensors):
+            if events is not None:
+                events[i][0].record()
+            step_fn(p, st, 1e-4, 0.01, 0.9, 0.999, 1e-8, step_no,
+                    decoupled_weight_decay=True, clip_coef=clip, **kw)
+            if events is not None:
+                events[i][1].record()
+
+    for w in range(args.warmup):
+        one_step(w + 1)
+    torch.cuda.synchronize()
+
+    # Timed region: exactly --steps steps, bracketed by device synchronisation.
+    use_events = not args.no_events
+    ev = None
+    kernel_ms = 0.0
+    launches = 0
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        if use_events:
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                  for _ in tensors]
+        one_step(args.warmup + s + 1, ev)
+        if use_events:
+            torch.cuda.synchronize()
+            kernel_ms += sum(a.elapsed_time(b) for a, b in ev)
+            launches += len(ev)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    ms_per_step = elapsed / args.steps * 1e3
+    value = bytes_per_step * args.steps / elapsed / 1e9
+
+    roofline = None
+    if use_events and launches:
+        avg_launch_s = kernel_ms / launches / 1e3
+        alg_bytes_per_launch = bytes_per_step / len(tensors)
+        achieved = alg_bytes_per_launch / avg_launch_s / 1e9
+        roofline = {
+            "bound": "hbm",
+            "kernel": f"adam_vec_kernel<{mode}>",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "alg_bytes_per_launch": int(alg_bytes_per_launch),
+            "avg_launch_us": round(avg_launch_s * 1e6, 2),
+            "launches": launches,
+        }
+
+    out = {
+        "metric": "fused Adam GB/s & % HBM peak; 8B offloaded step time (s), 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload,
+            "mode": mode,
+            "tensors": len(tensors),
+            "elements": total_elems,
+            "alg_bytes_per_elem": BYTES_PER_ELEM[mode],
+            "resident": "HBM",
+            "rng": kw.get("rng", "x8") if mode == "stochastic_rounding" else None,
+        },
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(mode)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

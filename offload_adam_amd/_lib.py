@@ -1,0 +1,94 @@
+"""ctypes binding of liboffload_adam_hip.so (the C ABI in include/offload_adam_hip.h).
+
+The library is loaded lazily on first use.  There is no fallback: if the
+shared object has not been built, every operator raises.
+"""
+
+import ctypes
+import threading
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint64, c_void_p
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "liboffload_adam_hip.so"
+
+OA_RNG_TRITON = 0
+OA_RNG_X8 = 1
+OA_RNG_BUFFER = 2
+
+_ADAM_TAIL = [c_int64, c_float, c_float, c_float, c_float, c_float, c_int]
+
+# name -> (restype, argtypes); every symbol include/offload_adam_hip.h declares.
+SIGNATURES = {
+    "oa_abi_version": (c_int, []),
+    "oa_error_string": (c_char_p, [c_int]),
+    "oa_adam_fp32_master": (
+        c_int,
+        [c_void_p] * 5 + _ADAM_TAIL + [c_void_p, c_void_p],
+    ),
+    "oa_adam_stochastic_rounding": (
+        c_int,
+        [c_void_p] * 4 + _ADAM_TAIL + [c_uint64, c_int, c_void_p, c_void_p, c_void_p],
+    ),
+    "oa_adam_fp31_master": (
+        c_int,
+        [c_void_p] * 5 + _ADAM_TAIL + [c_void_p, c_void_p],
+    ),
+    "oa_adam_fp32_master_custom_rounding": (
+        c_int,
+        [c_void_p] * 5 + _ADAM_TAIL + [c_void_p, c_void_p],
+    ),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+class LibraryNotBuiltError(RuntimeError):
+    pass
+
+
+def load():
+    """Return the loaded library (thread-safe; hooks call from the autograd thread)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise LibraryNotBuiltError(
+                f"{LIB_PATH} is missing. Build it with "
+                "`python -m offload_adam_amd._build` (needs ROCm hipcc); there is "
+                "no CPU or PyTorch fallback for the optimizer kernels."
+            )
+        lib = ctypes.CDLL(str(LIB_PATH), mode=ctypes.RTLD_LOCAL)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        built = lib.oa_abi_version()
+        if built != 1:
+            raise RuntimeError(f"{LIB_PATH} has ABI version {built}, expected 1")
+        _lib = lib
+    return _lib
+
+
+def error_string(code):
+    return load().oa_error_string(code).decode()
+
+
+def check(code, what):
+    """Raise RuntimeError for a non-zero return code of an entry point."""
+    if code != 0:
+        raise RuntimeError(f"{what} failed with code {code}: {error_string(code)}")
+
+
+def current_stream_ptr():
+    import torch
+
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t):
+    """Device/host address of a tensor's first element, or NULL for None."""
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(None)

@@ -1,0 +1,462 @@
+// Fused AdamW update kernels for gfx950 (MI355X) and their C entry points.
+//
+// One launch per parameter, one pass over HBM: every lane moves 8 consecutive
+// elements per array with 128-bit loads/stores (a wave reads 1 KiB contiguous
+// per array), does the whole update in registers and writes the results back.
+// No LDS, no matrix cores: the work is elementwise and HBM-bound
+// (14-20 bytes per element).
+//
+// Arithmetic contract (what the reference's Triton kernels compute,
+// src/offload_adam/kernels/*.py): fp32, one rounding per operation, correctly
+// rounded sqrt and divide, denormals kept, bf16 stores round to nearest even.
+
+#include "oa_common.hpp"
+
+#pragma clang fp contract(off)
+
+#ifndef OA_ADAM_THREADS
+#define OA_ADAM_THREADS 256
+#endif
+#ifndef OA_ADAM_UNROLL
+#define OA_ADAM_UNROLL 1
+#endif
+#ifndef OA_ADAM_NT_LD
+#define OA_ADAM_NT_LD 1
+#endif
+#ifndef OA_ADAM_NT_ST
+#define OA_ADAM_NT_ST 1
+#endif
+
+namespace oa {
+namespace {
+
+enum Mode : int { kFp32Master = 0, kStochastic = 1, kFp31 = 2, kCustom = 3 };
+
+struct AdamArgs {
+  uint16_t* p;        // bf16 param (fp32_master: write-only sink)
+  const uint16_t* g;  // bf16 grad, read-only
+  uint16_t* m;        // bf16 exp_avg
+  uint16_t* v;        // bf16 exp_avg_sq
+  void* aux;          // f32 master | i16 rounding_error | nullptr
+  const uint16_t* rand16;
+  const uint16_t* clip;  // one bf16 scalar or nullptr
+  int64_t n;
+  float lr, wd, lr_wd, omb1, omb2, eps;
+  uint32_t k0, k1;  // Philox key = (seed_lo, seed_hi)
+};
+
+template <typename T>
+__device__ __forceinline__ T ld(const T* p) {
+#if OA_ADAM_NT_LD
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
+template <typename T>
+__device__ __forceinline__ void st(T* p, T x) {
+#if OA_ADAM_NT_ST
+  __builtin_nontemporal_store(x, p);
+#else
+  *p = x;
+#endif
+}
+
+// The 16 random bits of element i under a Philox layout.
+template <int RNG>
+__device__ __forceinline__ uint32_t rand16_of(int64_t i, const AdamArgs& a) {
+  if (RNG == OA_RNG_TRITON) {
+    Philox r = philox4x32_10((uint32_t)i, (uint32_t)((uint64_t)i >> 32), 0u, 0u,
+                             a.k0, a.k1);
+    return r.c0 & 0xFFFFu;
+  } else if (RNG == OA_RNG_X8) {
+    const uint64_t j = (uint64_t)i >> 3;
+    Philox r = philox4x32_10((uint32_t)j, (uint32_t)(j >> 32), 1u, 0u, a.k0, a.k1);
+    const uint32_t e = (uint32_t)i & 7u;
+    const uint32_t w = (e >> 1) == 0 ? r.c0 : (e >> 1) == 1 ? r.c1
+                       : (e >> 1) == 2 ? r.c2 : r.c3;
+    return (w >> ((e & 1u) * 16u)) & 0xFFFFu;
+  } else {
+    return a.rand16[i];
+  }
+}
+
+// One element.  `pb` = bf16 bits of the param, `mb`/`vb` = bf16 bits of the
+// moments, `aux` = fp32 master bits or the int16 rounding error (low 16 bits).
+template <int MODE, bool DEC, bool CLIP>
+__device__ __forceinline__ void adam_elem(uint32_t& pb, uint32_t gb, float& m,
+                                          float& v, uint32_t& aux, uint32_t r16,
+                                          float clip, const AdamArgs& a) {
+  float g = bf16_bits_to_f32(gb);
+  if (CLIP) g = bf16_bits_to_f32(f32_to_bf16_1(g * clip));
+
+  float M;
+  if (MODE == kFp32Master) {
+    M = __uint_as_float(aux);
+  } else if (MODE == kStochastic) {
+    M = bf16_bits_to_f32(pb);
+  } else if (MODE == kFp31) {
+    const int32_t e = (int32_t)(int16_t)aux;
+    M = __uint_as_float((pb << 16) + ((uint32_t)e << 1));
+  } else {
+    const int32_t e = (int32_t)(int16_t)aux;
+    M = __uint_as_float((pb << 16) + (uint32_t)e);
+  }
+
+  if (DEC) {
+    M = M - a.lr_wd * M;
+  } else {
+    g = g + a.wd * M;
+  }
+  m = m + a.omb1 * (g - m);
+  v = v + a.omb2 * (g * g - v);
+  const float denom = sqrtf(v) + a.eps;
+  M = M - (a.lr * m) / denom;
+
+  const uint32_t x = __float_as_uint(M);
+  if (MODE == kFp32Master) {
+    aux = x;  // the caller stores bf16_rne(M) as the param
+  } else if (MODE == kStochastic) {
+    const uint32_t frac = x & 0xFFFFu;
+    const uint32_t trunc = x & 0xFFFF0000u;
+    pb = ((r16 < frac) ? trunc + 0x10000u : trunc) >> 16;
+  } else if (MODE == kFp31) {
+    // round to 31 bits, ties to even on bit 0 (arithmetic shifts)
+    const int32_t xi = (int32_t)x;
+    const int32_t up = xi & (xi >> 1) & 1;
+    const uint32_t x31 = (uint32_t)((xi >> 1) + up) << 1;
+    pb = f32_to_bf16_1(__uint_as_float(x31));
+    const int32_t err = (int32_t)(x31 - (pb << 16));
+    aux = (uint32_t)(err >> 1) & 0xFFFFu;
+  } else {
+    const int32_t xi = (int32_t)x;
+    pb = (uint32_t)((xi + 0x8000) >> 16) & 0xFFFFu;
+    aux = (x - (pb << 16)) & 0xFFFFu;
+  }
+}
+
+// Scalar path: one element per lane per trip.  Used for buffers that are not
+// 16-byte aligned and for the (n % 8) tail of the vector kernel.
+template <int MODE, bool DEC, bool CLIP, int RNG>
+__device__ __forceinline__ void adam_scalar(int64_t i, float clip,
+                                            const AdamArgs& a) {
+  uint32_t pb = (MODE == kFp32Master) ? 0u : a.p[i];
+  const uint32_t gb = a.g[i];
+  float m = bf16_bits_to_f32(a.m[i]);
+  float v = bf16_bits_to_f32(a.v[i]);
+  uint32_t aux = 0;
+  if (MODE == kFp32Master) aux = reinterpret_cast<const uint32_t*>(a.aux)[i];
+  if (MODE == kFp31 || MODE == kCustom)
+    aux = reinterpret_cast<const uint16_t*>(a.aux)[i];
+  uint32_t r16 = 0;
+  if (MODE == kStochastic) r16 = rand16_of<RNG>(i, a);
+  adam_elem<MODE, DEC, CLIP>(pb, gb, m, v, aux, r16, clip, a);
+  if (MODE == kFp32Master) pb = f32_to_bf16_1(__uint_as_float(aux));
+  a.p[i] = (uint16_t)pb;
+  a.m[i] = (uint16_t)f32_to_bf16_1(m);
+  a.v[i] = (uint16_t)f32_to_bf16_1(v);
+  if (MODE == kFp32Master) reinterpret_cast<uint32_t*>(a.aux)[i] = aux;
+  if (MODE == kFp31 || MODE == kCustom)
+    reinterpret_cast<uint16_t*>(a.aux)[i] = (uint16_t)aux;
+}
+
+template <int MODE, bool DEC, bool CLIP, int RNG>
+__global__ void __launch_bounds__(OA_ADAM_THREADS)
+adam_scalar_kernel(const AdamArgs a) {
+  const float clip = CLIP ? bf16_bits_to_f32(*a.clip) : 1.0f;
+  const int64_t stride = (int64_t)gridDim.x * OA_ADAM_THREADS;
+  for (int64_t i = (int64_t)blockIdx.x * OA_ADAM_THREADS + threadIdx.x; i < a.n;
+       i += stride)
+    adam_scalar<MODE, DEC, CLIP, RNG>(i, clip, a);
+}
+
+// Vector path.  A "group" is 8 consecutive elements.  Block b owns groups
+// [b*T*U, (b+1)*T*U); lane t takes groups b*T*U + k*T + t for k < U, so each
+// wave touches 1 KiB of consecutive bytes per array per k.  All loads of the
+// U groups are issued before any arithmetic to keep many bytes in flight.
+// 16-bit arrays travel as four packed dwords (element 2j in the low half of
+// dword j), which is also the layout the hardware bf16 convert produces.
+template <int MODE, bool DEC, bool CLIP, int RNG>
+__global__ void __launch_bounds__(OA_ADAM_THREADS)
+adam_vec_kernel(const AdamArgs a) {
+  constexpr int T = OA_ADAM_THREADS;
+  constexpr int U = OA_ADAM_UNROLL;
+  const int64_t n_groups = a.n >> 3;
+  const float clip = CLIP ? bf16_bits_to_f32(*a.clip) : 1.0f;
+  const int64_t g0 = (int64_t)blockIdx.x * (T * U) + threadIdx.x;
+
+  u32x4 P[U], G[U], Mo[U], Vo[U], R[U], E[U];
+  f32x4 Ma[U], Mb[U];
+  bool live[U];
+
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t grp = g0 + (int64_t)k * T;
+    live[k] = grp < n_groups;
+    if (live[k]) {
+      const int64_t e0 = grp << 3;
+      if (MODE != kFp32Master) P[k] = ld(reinterpret_cast<const u32x4*>(a.p + e0));
+      G[k] = ld(reinterpret_cast<const u32x4*>(a.g + e0));
+      Mo[k] = ld(reinterpret_cast<const u32x4*>(a.m + e0));
+      Vo[k] = ld(reinterpret_cast<const u32x4*>(a.v + e0));
+      if (MODE == kFp32Master) {
+        const float* mp = reinterpret_cast<const float*>(a.aux) + e0;
+        Ma[k] = ld(reinterpret_cast<const f32x4*>(mp));
+        Mb[k] = ld(reinterpret_cast<const f32x4*>(mp + 4));
+      }
+      if (MODE == kFp31 || MODE == kCustom)
+        E[k] = ld(reinterpret_cast<const u32x4*>(
+            reinterpret_cast<const uint16_t*>(a.aux) + e0));
+      if (MODE == kStochastic && RNG == OA_RNG_BUFFER)
+        R[k] = ld(reinterpret_cast<const u32x4*>(a.rand16 + e0));
+    }
+  }
+
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    if (!live[k]) continue;
+    const int64_t grp = g0 + (int64_t)k * T;
+    const int64_t e0 = grp << 3;
+
+    u32x4 RW = {0u, 0u, 0u, 0u};
+    if (MODE == kStochastic && RNG == OA_RNG_X8) {
+      Philox r = philox4x32_10((uint32_t)grp, (uint32_t)((uint64_t)grp >> 32), 1u,
+                               0u, a.k0, a.k1);
+      RW = u32x4{r.c0, r.c1, r.c2, r.c3};
+    }
+    if (MODE == kStochastic && RNG == OA_RNG_BUFFER) RW = R[k];
+
+    u32x4 Pn, Mn, Vn, En;
+    f32x4 Mlo, Mhi;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t pb[2], ax[2];
+      float m[2], v[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int e = 2 * j + h;
+        const uint32_t sh = h * 16;
+        pb[h] = (MODE == kFp32Master) ? 0u : ((P[k][j] >> sh) & 0xFFFFu);
+        const uint32_t gb = (G[k][j] >> sh) & 0xFFFFu;
+        m[h] = h ? bf16hi_to_f32(Mo[k][j]) : bf16lo_to_f32(Mo[k][j]);
+        v[h] = h ? bf16hi_to_f32(Vo[k][j]) : bf16lo_to_f32(Vo[k][j]);
+        ax[h] = 0;
+        if (MODE == kFp32Master)
+          ax[h] = __float_as_uint(e < 4 ? Ma[k][e & 3] : Mb[k][e & 3]);
+        if (MODE == kFp31 || MODE == kCustom) ax[h] = (E[k][j] >> sh) & 0xFFFFu;
+        uint32_t r16 = 0;
+        if (MODE == kStochastic) {
+          if (RNG == OA_RNG_TRITON) {
+            const int64_t i = e0 + e;
+            Philox r = philox4x32_10((uint32_t)i, (uint32_t)((uint64_t)i >> 32),
+                                     0u, 0u, a.k0, a.k1);
+            r16 = r.c0 & 0xFFFFu;
+          } else {
+            r16 = (RW[j] >> sh) & 0xFFFFu;
+          }
+        }
+        adam_elem<MODE, DEC, CLIP>(pb[h], gb, m[h], v[h], ax[h], r16, clip, a);
+      }
+      Mn[j] = f32x2_to_bf16x2_bits(m[0], m[1]);
+      Vn[j] = f32x2_to_bf16x2_bits(v[0], v[1]);
+      if (MODE == kFp32Master) {
+        const float M0 = __uint_as_float(ax[0]), M1 = __uint_as_float(ax[1]);
+        Pn[j] = f32x2_to_bf16x2_bits(M0, M1);
+        if (j < 2) {
+          Mlo[2 * j] = M0;
+          Mlo[2 * j + 1] = M1;
+        } else {
+          Mhi[2 * j - 4] = M0;
+          Mhi[2 * j - 3] = M1;
+        }
+      } else {
+        Pn[j] = pb[0] | (pb[1] << 16);
+      }
+      if (MODE == kFp31 || MODE == kCustom) En[j] = ax[0] | (ax[1] << 16);
+    }
+
+    st(reinterpret_cast<u32x4*>(a.m + e0), Mn);
+    st(reinterpret_cast<u32x4*>(a.v + e0), Vn);
+    st(reinterpret_cast<u32x4*>(a.p + e0), Pn);
+    if (MODE == kFp32Master) {
+      float* mp = reinterpret_cast<float*>(a.aux) + e0;
+      st(reinterpret_cast<f32x4*>(mp), Mlo);
+      st(reinterpret_cast<f32x4*>(mp + 4), Mhi);
+    }
+    if (MODE == kFp31 || MODE == kCustom)
+      st(reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.aux) + e0), En);
+  }
+
+  // Tail: the last n % 8 elements, one lane each, in the last block.
+  if (blockIdx.x == gridDim.x - 1) {
+    const int64_t i = (n_groups << 3) + threadIdx.x;
+    if (i < a.n) adam_scalar<MODE, DEC, CLIP, RNG>(i, clip, a);
+  }
+}
+
+template <int MODE, bool DEC, bool CLIP, int RNG>
+int launch(const AdamArgs& a, bool vec, hipStream_t s) {
+  constexpr int T = OA_ADAM_THREADS;
+  if (vec) {
+    const int64_t per_block = (int64_t)T * OA_ADAM_UNROLL * 8;
+    int64_t blocks = (a.n + per_block - 1) / per_block;
+    if (blocks > 0x7FFFFFFFll) return OA_ERANGE;
+    hipLaunchKernelGGL((adam_vec_kernel<MODE, DEC, CLIP, RNG>), dim3((unsigned)blocks),
+                       dim3(T), 0, s, a);
+  } else {
+    int64_t blocks = (a.n + T - 1) / T;
+    if (blocks > 65536) blocks = 65536;  // grid-stride beyond this
+    hipLaunchKernelGGL((adam_scalar_kernel<MODE, DEC, CLIP, RNG>),
+                       dim3((unsigned)blocks), dim3(T), 0, s, a);
+  }
+  return launch_status();
+}
+
+template <int MODE, int RNG>
+int dispatch_flags(const AdamArgs& a, bool dec, bool vec, hipStream_t s) {
+  const bool clip = a.clip != nullptr;
+  if (dec) {
+    return clip ? launch<MODE, true, true, RNG>(a, vec, s)
+                : launch<MODE, true, false, RNG>(a, vec, s);
+  }
+  return clip ? launch<MODE, false, true, RNG>(a, vec, s)
+              : launch<MODE, false, false, RNG>(a, vec, s);
+}
+
+// Argument checks shared by the four entry points.  Returns 0, or an OA_E*.
+int check_common(const void* p, const void* g, const void* m, const void* v,
+                 const void* aux, bool has_aux, size_t aux_align, int64_t n,
+                 const void* clip, bool p_may_alias_g) {
+  if (n < 0) return OA_EINVAL;
+  if (n == 0) return 0;
+  if (!p || !g || !m || !v || (has_aux && !aux)) return OA_EINVAL;
+  if (!aligned_to(p, 2) || !aligned_to(g, 2) || !aligned_to(m, 2) ||
+      !aligned_to(v, 2) || (has_aux && !aligned_to(aux, aux_align)) ||
+      (clip && !aligned_to(clip, 2)))
+    return OA_EALIGN;
+  // Buffers that are written must be pairwise distinct, and distinct from grad.
+  const void* w[4] = {p, m, v, has_aux ? aux : nullptr};
+  for (int i = 0; i < 4; ++i) {
+    if (!w[i]) continue;
+    for (int j = i + 1; j < 4; ++j)
+      if (w[j] && w[i] == w[j]) return OA_EOVERLAP;
+    if (w[i] == g && !(i == 0 && p_may_alias_g)) return OA_EOVERLAP;
+  }
+  return 0;
+}
+
+AdamArgs make_args(void* p, const void* g, void* m, void* v, void* aux,
+                   int64_t n, float lr, float wd, float b1h, float b2h, float eps,
+                   const void* clip) {
+  AdamArgs a;
+  a.p = static_cast<uint16_t*>(p);
+  a.g = static_cast<const uint16_t*>(g);
+  a.m = static_cast<uint16_t*>(m);
+  a.v = static_cast<uint16_t*>(v);
+  a.aux = aux;
+  a.rand16 = nullptr;
+  a.clip = static_cast<const uint16_t*>(clip);
+  a.n = n;
+  a.lr = lr;
+  a.wd = wd;
+  // Scalar sub-expressions of the update, each a single fp32 operation: the
+  // same values the kernel would compute per element.
+  volatile float lr_wd = lr * wd;
+  volatile float omb1 = 1.0f - b1h;
+  volatile float omb2 = 1.0f - b2h;
+  a.lr_wd = lr_wd;
+  a.omb1 = omb1;
+  a.omb2 = omb2;
+  a.eps = eps;
+  a.k0 = a.k1 = 0;
+  return a;
+}
+
+bool all16(const void* p, const void* g, const void* m, const void* v,
+           const void* aux, const void* r) {
+  return aligned_to(p, 16) && aligned_to(g, 16) && aligned_to(m, 16) &&
+         aligned_to(v, 16) && (!aux || aligned_to(aux, 16)) &&
+         (!r || aligned_to(r, 16));
+}
+
+}  // namespace
+}  // namespace oa
+
+using namespace oa;
+
+extern "C" int oa_adam_fp32_master(void* param_out, const void* grad, void* exp_avg,
+                                   void* exp_avg_sq, void* master, int64_t n,
+                                   float lr, float weight_decay, float beta1_hat,
+                                   float beta2_hat, float eps, int decoupled,
+                                   const void* clip_coef, void* stream) {
+  int rc = check_common(param_out, grad, exp_avg, exp_avg_sq, master, true, 4, n,
+                        clip_coef, /*p_may_alias_g=*/true);
+  if (rc != 0 || n == 0) return rc;
+  AdamArgs a = make_args(param_out, grad, exp_avg, exp_avg_sq, master, n, lr,
+                         weight_decay, beta1_hat, beta2_hat, eps, clip_coef);
+  const bool vec = all16(param_out, grad, exp_avg, exp_avg_sq, master, nullptr);
+  return dispatch_flags<kFp32Master, OA_RNG_TRITON>(a, decoupled != 0, vec,
+                                                    static_cast<hipStream_t>(stream));
+}
+
+extern "C" int oa_adam_stochastic_rounding(void* param, const void* grad,
+                                           void* exp_avg, void* exp_avg_sq,
+                                           int64_t n, float lr, float weight_decay,
+                                           float beta1_hat, float beta2_hat,
+                                           float eps, int decoupled, uint64_t seed,
+                                           int rng, const void* rand16,
+                                           const void* clip_coef, void* stream) {
+  if (rng != OA_RNG_TRITON && rng != OA_RNG_X8 && rng != OA_RNG_BUFFER)
+    return OA_EINVAL;
+  int rc = check_common(param, grad, exp_avg, exp_avg_sq, nullptr, false, 1, n,
+                        clip_coef, false);
+  if (rc != 0 || n == 0) return rc;
+  if (rng == OA_RNG_BUFFER) {
+    if (!rand16) return OA_EINVAL;
+    if (!aligned_to(rand16, 2)) return OA_EALIGN;
+  }
+  AdamArgs a = make_args(param, grad, exp_avg, exp_avg_sq, nullptr, n, lr,
+                         weight_decay, beta1_hat, beta2_hat, eps, clip_coef);
+  a.k0 = (uint32_t)(seed & 0xFFFFFFFFull);
+  a.k1 = (uint32_t)(seed >> 32);
+  a.rand16 = static_cast<const uint16_t*>(rand16);
+  const bool vec = all16(param, grad, exp_avg, exp_avg_sq, nullptr,
+                         rng == OA_RNG_BUFFER ? rand16 : nullptr);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool dec = decoupled != 0;
+  if (rng == OA_RNG_TRITON)
+    return dispatch_flags<kStochastic, OA_RNG_TRITON>(a, dec, vec, s);
+  if (rng == OA_RNG_X8) return dispatch_flags<kStochastic, OA_RNG_X8>(a, dec, vec, s);
+  return dispatch_flags<kStochastic, OA_RNG_BUFFER>(a, dec, vec, s);
+}
+
+extern "C" int oa_adam_fp31_master(void* param, const void* grad, void* exp_avg,
+                                   void* exp_avg_sq, void* rounding_error,
+                                   int64_t n, float lr, float weight_decay,
+                                   float beta1_hat, float beta2_hat, float eps,
+                                   int decoupled, const void* clip_coef,
+                                   void* stream) {
+  int rc = check_common(param, grad, exp_avg, exp_avg_sq, rounding_error, true, 2,
+                        n, clip_coef, false);
+  if (rc != 0 || n == 0) return rc;
+  AdamArgs a = make_args(param, grad, exp_avg, exp_avg_sq, rounding_error, n, lr,
+                         weight_decay, beta1_hat, beta2_hat, eps, clip_coef);
+  const bool vec = all16(param, grad, exp_avg, exp_avg_sq, rounding_error, nullptr);
+  return dispatch_flags<kFp31, OA_RNG_TRITON>(a, decoupled != 0, vec,
+                                              static_cast<hipStream_t>(stream));
+}
+
+extern "C" int oa_adam_fp32_master_custom_rounding(
+    void* param, const void* grad, void* exp_avg, void* exp_avg_sq,
+    void* rounding_error, int64_t n, float lr, float weight_decay, float beta1_hat,
+    float beta2_hat, float eps, int decoupled, const void* clip_coef,
+    void* stream) {
+  int rc = check_common(param, grad, exp_avg, exp_avg_sq, rounding_error, true, 2,
+                        n, clip_coef, false);
+  if (rc != 0 || n == 0) return rc;
+  AdamArgs a = make_args(param, grad, exp_avg, exp_avg_sq, rounding_error, n, lr,
+                         weight_decay, beta1_hat, beta2_hat, eps, clip_coef);
+  const bool vec = all16(param, grad, exp_avg, exp_avg_sq, rounding_error, nullptr);
+  return dispatch_flags<kCustom, OA_RNG_TRITON>(a, decoupled != 0, vec,
+                                                static_cast<hipStream_t>(stream));
+}

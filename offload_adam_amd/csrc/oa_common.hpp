@@ -1,0 +1,100 @@
+// Shared device/host helpers of liboffload_adam_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "offload_adam_hip.h"
+
+// Every floating-point expression in this library is evaluated exactly as
+// written: one IEEE rounding per operation, never contracted into an FMA.
+#pragma clang fp contract(off)
+
+namespace oa {
+
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned char u8x16 __attribute__((ext_vector_type(16)));
+typedef unsigned char u8x8 __attribute__((ext_vector_type(8)));
+typedef unsigned char u8x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) {
+  return __uint_as_float(h << 16);
+}
+
+// Two fp32 -> packed bf16x2 (lo in bits 0..15) through the gfx950 hardware
+// convert (v_cvt_pk_bf16_f32): round to nearest even, NaN stays a quiet NaN.
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  f32x2 in = {lo, hi};
+  bf16x2_t out = __builtin_convertvector(in, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, out);
+}
+
+// One fp32 -> bf16 bits (in the low 16 bits of the result).
+__device__ __forceinline__ uint32_t f32_to_bf16_1(float f) {
+  return f32x2_to_bf16x2_bits(f, 0.0f) & 0xFFFFu;
+}
+
+// Low / high bf16 half of a packed dword, widened to fp32.
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t w) {
+  return __uint_as_float(w << 16);
+}
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t w) {
+  return __uint_as_float(w & 0xFFFF0000u);
+}
+
+// Philox4x32-10 (Salmon et al., SC'11): round multipliers 0xD2511F53 and
+// 0xCD9E8D57, key increments 0x9E3779B9 and 0xBB67AE85.
+struct Philox {
+  uint32_t c0, c1, c2, c3;
+};
+
+__device__ __forceinline__ Philox philox4x32_10(uint32_t c0, uint32_t c1,
+                                                uint32_t c2, uint32_t c3,
+                                                uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t pb = (uint64_t)0xCD9E8D57u * (uint64_t)c2;
+    const uint64_t pa = (uint64_t)0xD2511F53u * (uint64_t)c0;
+    const uint32_t n0 = (uint32_t)(pb >> 32) ^ c1 ^ k0;
+    const uint32_t n2 = (uint32_t)(pa >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)pb;
+    c3 = (uint32_t)pa;
+    c0 = n0;
+    c2 = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return Philox{c0, c1, c2, c3};
+}
+
+// Wave64 all-lane sum via butterfly shuffles (every lane ends with the total).
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) x += __shfl_xor(x, off, kWave);
+  return x;
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1)
+    x = fmaxf(x, __shfl_xor(x, off, kWave));
+  return x;
+}
+
+inline bool aligned_to(const void* p, uintptr_t a) {
+  return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+inline int launch_status() { return static_cast<int>(hipGetLastError()); }
+
+}  // namespace oa

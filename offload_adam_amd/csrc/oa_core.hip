@@ -1,0 +1,26 @@
+// Version and error-text entry points of liboffload_adam_hip.so.
+#include "oa_common.hpp"
+
+extern "C" int oa_abi_version(void) { return OA_ABI_VERSION; }
+
+extern "C" const char* oa_error_string(int code) {
+  switch (code) {
+    case 0:
+      return "success";
+    case OA_EINVAL:
+      return "offload_adam_hip: invalid argument (null pointer, negative size or bad enum)";
+    case OA_EALIGN:
+      return "offload_adam_hip: pointer is not aligned to its element type";
+    case OA_ERANGE:
+      return "offload_adam_hip: size is beyond what this entry point supports";
+    case OA_EOVERLAP:
+      return "offload_adam_hip: buffers that must be distinct alias each other";
+    default:
+      break;
+  }
+  if (code > 0) {
+    const char* s = hipGetErrorString(static_cast<hipError_t>(code));
+    return s ? s : "offload_adam_hip: unknown HIP error";
+  }
+  return "offload_adam_hip: unknown error code";
+}
