@@ -132,6 +132,115 @@ int oa_adam_fp32_master_custom_rounding(void* param, const void* grad,
                                         float eps, int decoupled,
                                         const void* clip_coef, void* stream);
 
+/* ------------------------------------------------------------------------
+ * B. Gradient L2 norm per parameter and the global clip coefficient.
+ * ---------------------------------------------------------------------- */
+
+/* Bytes of device scratch oa_grad_norm_bf16 needs.  The caller allocates it
+ * (64-byte aligned), zero-fills it ONCE, and may reuse it for every later call
+ * on the same stream: each launch leaves it zeroed again.  Launches that may
+ * overlap (different streams) need separate workspaces. */
+size_t oa_norm_workspace_bytes(void);
+
+/* Replaces `torch.norm(grad, 2.0)` on the accumulated bf16 gradient
+ * (src/offload_adam/offload_adam.py:504-505, 531-532).
+ *   grad       bf16[n], any 2-byte alignment
+ *   norm_out   ONE bf16: bf16_rne(sqrt(sum g^2)), fp32 accumulation in a fixed
+ *              order (bit-reproducible run to run)
+ *   sumsq_out  NULL or ONE f32 receiving the unrounded sum of squares */
+int oa_grad_norm_bf16(const void* grad, int64_t n, void* norm_out, void* sumsq_out,
+                      void* workspace, void* stream);
+
+/* Replaces the global-norm and clip-coefficient arithmetic of
+ * OffloadAdam.step (src/offload_adam/offload_adam.py:553-561):
+ *   total = vector_norm(stack(norms), 2)                        (bf16)
+ *   coef  = clamp(max_norm / (total + 1e-6), max=1.0)           (bf16)
+ * with torch's evaluation of `float / tensor` as reciprocal()*float, every
+ * step rounded to bf16 like the 0-dim bf16 tensor ops do.  No host sync.
+ *   norms      bf16[count] (the per-parameter norms, contiguous)
+ *   total_out  NULL or ONE bf16;  coef_out  ONE bf16 */
+int oa_clip_coef_bf16(const void* norms, int64_t count, float max_norm,
+                      void* total_out, void* coef_out, void* stream);
+
+/* ------------------------------------------------------------------------
+ * C. Weight-only quantisation codecs for (rows = out_features, cols =
+ *    in_features) matrices.  `src`/`out` are row-major with unit column stride
+ *    and a row stride given in ELEMENTS; packed payloads are contiguous.
+ *    Element types of float operands: */
+#define OA_F32  0
+#define OA_BF16 1
+#define OA_F16  2
+/*    Quantise entry points read the source once per output (the amax passes
+ *    hit the same data again through L2 / registers) and write straight into
+ *    the payload buffers of the quantised weight.  Results are bit-identical
+ *    to the reference's pure-torch functions named at each entry point. */
+
+/* int8, per-row symmetric.  Replaces _quantize_int8_triton
+ * (src/offload_adam/qweight/int8.py:202-232; spec: quantize_int8_per_channel,
+ * int8.py:30-49).  q: int8[rows*cols]; scales: [rows] of scale_dtype
+ * (scale = absmax/127 rounded to scale_dtype; the codes use the fp32 scale). */
+int oa_quant_int8(const void* src, int src_dtype, int64_t src_row_stride,
+                  int64_t rows, int64_t cols, void* q, void* scales,
+                  int scale_dtype, void* stream);
+
+/* Replaces _dequant_int8_triton (int8.py:107-126; spec:
+ * dequantize_int8_per_channel, int8.py:52-57): out = round(q * scale) in
+ * out_dtype, with the stored scale widened from scale_dtype. */
+int oa_dequant_int8(const void* q, const void* scales, int scale_dtype,
+                    int64_t rows, int64_t cols, void* out, int out_dtype,
+                    int64_t out_row_stride, void* stream);
+
+/* int4, symmetric, groups of `group` columns, GPTQ storage.  Replaces
+ * _quantize_pack_int4_triton (src/offload_adam/qweight/int4.py:258-296; spec:
+ * quantize_int4_groupwise + pack_int4_gptq, int4.py:30-48, 61-92).
+ * qweight: int32[(cols/8) * rows], word (k, r) packs columns 8k..8k+7 of row r
+ * LSB first as (code + 8); scales: [(cols/group) * rows] of scale_dtype.
+ * cols % group == 0, group % 8 == 0. */
+int oa_quant_int4(const void* src, int src_dtype, int64_t src_row_stride,
+                  int64_t rows, int64_t cols, int64_t group, void* qweight,
+                  void* scales, int scale_dtype, void* stream);
+
+/* Replaces _dequant_int4_triton (int4.py:155-183). */
+int oa_dequant_int4(const void* qweight, const void* scales, int scale_dtype,
+                    int64_t rows, int64_t cols, int64_t group, void* out,
+                    int out_dtype, int64_t out_row_stride, void* stream);
+
+/* NF4, blocks of `block` columns, bitsandbytes storage.  Replaces
+ * _quantize_nf4_triton (src/offload_adam/qweight/nf4.py:334-372; spec:
+ * quantize_nf4_blockwise + pack_nf4, nf4.py:74-83, 102-135).
+ * packed: uint8[rows * cols/2], even column in the HIGH nibble;
+ * absmax: f32[rows * cols/block].  cols % block == 0, block % 2 == 0. */
+int oa_quant_nf4(const void* src, int src_dtype, int64_t src_row_stride,
+                 int64_t rows, int64_t cols, int64_t block, void* packed,
+                 void* absmax, void* stream);
+
+/* Replaces _dequant_nf4_triton (nf4.py:230-260): fp32 codebook value times
+ * fp32 absmax, rounded once to out_dtype. */
+int oa_dequant_nf4(const void* packed, const void* absmax, int64_t rows,
+                   int64_t cols, int64_t block, void* out, int out_dtype,
+                   int64_t out_row_stride, void* stream);
+
+/* NVFP4: e2m1 codes in blocks of 16 with float8_e4m3fn block scales and one
+ * fp32 tensor scale.  Replaces _quantize_nvfp4_triton
+ * (src/offload_adam/qweight/nvfp4.py:660-732; spec: quantize_nvfp4_blockwise +
+ * pack_fp4, nvfp4.py:72-81, 133-173).  Two launches: tensor amax, then encode.
+ *   packed        uint8[rows * cols/2], even column in the LOW nibble
+ *   block_scale   uint8[rows * cols/16], float8_e4m3fn bit patterns
+ *   global_scale  ONE f32 (device), written: max(amax,1e-12) / (448*6)
+ *   workspace     as for oa_grad_norm_bf16 (oa_norm_workspace_bytes() bytes,
+ *                 zero-filled once)
+ * cols % 16 == 0. */
+int oa_quant_nvfp4(const void* src, int src_dtype, int64_t src_row_stride,
+                   int64_t rows, int64_t cols, void* packed, void* block_scale,
+                   void* global_scale, void* workspace, void* stream);
+
+/* Replaces _dequant_nvfp4_triton (nvfp4.py:411-461, soft path): e2m1 value
+ * times (e4m3 scale * global scale) in fp32, rounded once to out_dtype. */
+int oa_dequant_nvfp4(const void* packed, const void* block_scale,
+                     const void* global_scale, int64_t rows, int64_t cols,
+                     void* out, int out_dtype, int64_t out_row_stride,
+                     void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -37,7 +37,65 @@ SIGNATURES = {
         c_int,
         [c_void_p] * 5 + _ADAM_TAIL + [c_void_p, c_void_p],
     ),
+    "oa_norm_workspace_bytes": (c_size_t, []),
+    "oa_grad_norm_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "oa_clip_coef_bf16": (
+        c_int,
+        [c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p],
+    ),
+    # src, src_dtype, stride, rows, cols, q, scales, scale_dtype, stream
+    "oa_quant_int8": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p],
+    ),
+    # q, scales, scale_dtype, rows, cols, out, out_dtype, out_stride, stream
+    "oa_dequant_int8": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p],
+    ),
+    "oa_quant_int4": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int,
+         c_void_p],
+    ),
+    "oa_dequant_int4": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64,
+         c_void_p],
+    ),
+    "oa_quant_nf4": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
+    "oa_dequant_nf4": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p],
+    ),
+    "oa_quant_nvfp4": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_void_p],
+    ),
+    "oa_dequant_nvfp4": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p],
+    ),
 }
+
+OA_F32, OA_BF16, OA_F16 = 0, 1, 2
+
+
+def dtype_code(dtype):
+    """torch float dtype -> OA_* element-type code of the C ABI."""
+    import torch
+
+    try:
+        return {torch.float32: OA_F32, torch.bfloat16: OA_BF16, torch.float16: OA_F16}[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype}; expected float32, bfloat16 or float16")
 
 _lib = None
 _lock = threading.Lock()

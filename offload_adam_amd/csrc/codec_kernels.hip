@@ -1,0 +1,923 @@
+// Weight-only quantisation codecs for gfx950: int8 per-row, int4 group-wise
+// (GPTQ layout), NF4 block-wise (bitsandbytes layout), NVFP4 (e2m1 codes,
+// float8_e4m3fn block scales, fp32 tensor scale).
+//
+// All kernels are HBM-bound byte shuffling: a lane owns an "octet" (8
+// consecutive columns of one row), loaded and stored with one or two 128-bit
+// accesses; group maxima are folded with wave64 sub-group shuffles; the int4
+// layout, which is stored transposed, goes through an LDS tile so that both the
+// row-major side and the column-major side are written in long runs.
+//
+// Arithmetic is fp32 with one rounding per operation (no FMA contraction,
+// correctly rounded divide), which makes the codes bit-identical to the
+// reference's pure-torch quantisers.
+//
+// Each codec has a fast path (cols % 8 == 0, 16-byte aligned rows, power-of-two
+// group) and a generic path (one lane per group, any shape and alignment).
+
+#include "oa_common.hpp"
+
+#pragma clang fp contract(off)
+
+namespace oa {
+namespace {
+
+constexpr int kT = 256;
+constexpr float kEps = 1e-12f;
+
+// ------------------------------------------------------------ element access
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  // The empty asm keeps the fp32 value as computed: without it the backend may
+  // merge a preceding fp32 multiply with this convert into one mixed-precision
+  // instruction that rounds the exact product straight to fp16 (one rounding
+  // instead of two), which differs at fp32 ties.
+  asm volatile("" : "+v"(f));
+  return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f);
+}
+
+template <int DT>
+__device__ __forceinline__ float load1(const void* base, int64_t i) {
+  if (DT == OA_F32) return static_cast<const float*>(base)[i];
+  const uint32_t h = static_cast<const uint16_t*>(base)[i];
+  return DT == OA_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+}
+
+// 8 consecutive elements starting at element i (16-byte aligned address).
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t i, float (&x)[8]) {
+  if (DT == OA_F32) {
+    const f32x4* p = reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + i);
+    const f32x4 a = p[0], b = p[1];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { x[k] = a[k]; x[4 + k] = b[k]; }
+  } else {
+    const u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + i);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (DT == OA_BF16) {
+        x[2 * k] = bf16lo_to_f32(w[k]);
+        x[2 * k + 1] = bf16hi_to_f32(w[k]);
+      } else {
+        x[2 * k] = f16_bits_to_f32(w[k] & 0xFFFFu);
+        x[2 * k + 1] = f16_bits_to_f32(w[k] >> 16);
+      }
+    }
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void store1(void* base, int64_t i, float v) {
+  if (DT == OA_F32) static_cast<float*>(base)[i] = v;
+  else if (DT == OA_BF16) static_cast<uint16_t*>(base)[i] = (uint16_t)f32_to_bf16_1(v);
+  else static_cast<uint16_t*>(base)[i] = (uint16_t)f32_to_f16_bits(v);
+}
+
+template <int DT>
+__device__ __forceinline__ void store8(void* base, int64_t i, const float (&x)[8]) {
+  if (DT == OA_F32) {
+    f32x4* p = reinterpret_cast<f32x4*>(static_cast<float*>(base) + i);
+    p[0] = f32x4{x[0], x[1], x[2], x[3]};
+    p[1] = f32x4{x[4], x[5], x[6], x[7]};
+  } else {
+    u32x4 w;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (DT == OA_BF16) w[k] = f32x2_to_bf16x2_bits(x[2 * k], x[2 * k + 1]);
+      else w[k] = f32_to_f16_bits(x[2 * k]) | (f32_to_f16_bits(x[2 * k + 1]) << 16);
+    }
+    *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base) + i) = w;
+  }
+}
+
+__device__ __forceinline__ float load_scale(const void* s, int dt, int64_t i) {
+  if (dt == OA_F32) return load1<OA_F32>(s, i);
+  if (dt == OA_BF16) return load1<OA_BF16>(s, i);
+  return load1<OA_F16>(s, i);
+}
+__device__ __forceinline__ void store_scale(void* s, int dt, int64_t i, float v) {
+  if (dt == OA_F32) store1<OA_F32>(s, i, v);
+  else if (dt == OA_BF16) store1<OA_BF16>(s, i, v);
+  else store1<OA_F16>(s, i, v);
+}
+
+__device__ __forceinline__ float absmax8(const float (&x)[8]) {
+  float a = 0.0f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) a = fmaxf(a, fabsf(x[k]));
+  return a;
+}
+
+// max over aligned sub-groups of `width` lanes (power of two <= 64)
+__device__ __forceinline__ float group_max(float a, int width) {
+  for (int off = width >> 1; off > 0; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, kWave));
+  return a;
+}
+
+__device__ __forceinline__ float block_max(float x, float* lds) {
+  x = wave_max(x);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = x;
+  __syncthreads();
+  float t = lds[0];
+#pragma unroll
+  for (int w = 1; w < kT / kWave; ++w) t = fmaxf(t, lds[w]);
+  __syncthreads();
+  return t;
+}
+
+// ------------------------------------------------------------------- int8
+
+__device__ __forceinline__ int32_t q_int8(float x, float inv) {
+  float t = __builtin_rintf(x * inv);
+  t = fminf(fmaxf(t, -128.0f), 127.0f);
+  return (int32_t)t;
+}
+
+// One block per row: pass 1 folds |x| into the row maximum, pass 2 re-reads the
+// row (L2-resident: a row is tens of KiB) and writes the codes.
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+quant_int8_kernel(const void* __restrict__ src, int64_t stride, int64_t cols,
+                  int8_t* __restrict__ q, void* __restrict__ scales, int sdt, int vec) {
+  __shared__ float lds[kT / kWave];
+  const int64_t row = blockIdx.x;
+  const int64_t base = row * stride;
+  const int64_t octets = vec ? cols >> 3 : 0;
+  float a = 0.0f;
+  for (int64_t o = threadIdx.x; o < octets; o += kT) {
+    float x[8];
+    load8<SRC>(src, base + o * 8, x);
+    a = fmaxf(a, absmax8(x));
+  }
+  for (int64_t c = octets * 8 + threadIdx.x; c < cols; c += kT)
+    a = fmaxf(a, fabsf(load1<SRC>(src, base + c)));
+  const float absmax = block_max(a, lds);
+  const float scale = absmax / 127.0f;
+  const float inv = 1.0f / fmaxf(scale, kEps);
+  if (threadIdx.x == 0) store_scale(scales, sdt, row, scale);
+
+  int8_t* qr = q + row * cols;
+  for (int64_t o = threadIdx.x; o < octets; o += kT) {
+    float x[8];
+    load8<SRC>(src, base + o * 8, x);
+    uint32_t w0 = 0, w1 = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      w0 |= ((uint32_t)q_int8(x[k], inv) & 0xFFu) << (8 * k);
+      w1 |= ((uint32_t)q_int8(x[4 + k], inv) & 0xFFu) << (8 * k);
+    }
+    *reinterpret_cast<u32x2*>(qr + o * 8) = u32x2{w0, w1};
+  }
+  for (int64_t c = octets * 8 + threadIdx.x; c < cols; c += kT)
+    qr[c] = (int8_t)q_int8(load1<SRC>(src, base + c), inv);
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(kT)
+dequant_int8_kernel(const int8_t* __restrict__ q, const void* __restrict__ scales, int sdt,
+                    int64_t rows, int64_t cols, void* __restrict__ out, int64_t ostride,
+                    int vec) {
+  if (vec) {
+    const int64_t opr = cols >> 3;
+    const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
+    if (o >= rows * opr) return;
+    const int64_t row = o / opr, c8 = o - row * opr;
+    const float s = load_scale(scales, sdt, row);
+    const u32x2 w = *reinterpret_cast<const u32x2*>(q + row * cols + c8 * 8);
+    float y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int32_t v = (int32_t)(int8_t)((w[k >> 2] >> (8 * (k & 3))) & 0xFFu);
+      y[k] = (float)v * s;
+    }
+    store8<OUT>(out, row * ostride + c8 * 8, y);
+  } else {
+    const int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x;
+    if (i >= rows * cols) return;
+    const int64_t row = i / cols, c = i - row * cols;
+    store1<OUT>(out, row * ostride + c, (float)q[i] * load_scale(scales, sdt, row));
+  }
+}
+
+// ------------------------------------------------------------------- int4
+
+__device__ __forceinline__ uint32_t q_int4_word(const float (&x)[8], float inv) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float t = __builtin_rintf(x[k] * inv);
+    t = fminf(fmaxf(t, -8.0f), 7.0f);
+    word |= (uint32_t)((int32_t)t + 8) << (4 * k);
+  }
+  return word;
+}
+
+constexpr int kI4Rows = 64;  // rows of one LDS tile
+
+// Block tile: 64 rows x one group.  WPR = group/8 lanes share a (row, group):
+// they fold the group maximum with shuffles and emit one packed word each into
+// LDS; the tile is then written with lanes running along the row index, which
+// is the contiguous direction of the transposed (cols/8, rows) storage.
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+quant_int4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int group,
+                  int32_t* __restrict__ qweight, void* __restrict__ scales, int sdt) {
+  extern __shared__ uint32_t i4_lds[];
+  const int wpr = group >> 3;
+  uint32_t* words = i4_lds;                                  // [wpr][kI4Rows + 1]
+  float* scale_s = reinterpret_cast<float*>(words + wpr * (kI4Rows + 1));
+  const int64_t r0 = (int64_t)blockIdx.x * kI4Rows;
+  const int64_t gi = blockIdx.y;
+  const int rows_per_pass = kT / wpr;
+  const int k = threadIdx.x % wpr;
+  for (int pr = 0; pr < kI4Rows; pr += rows_per_pass) {
+    const int rl = pr + threadIdx.x / wpr;
+    const int64_t row = r0 + rl;
+    float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (rl < kI4Rows && row < rows) load8<SRC>(src, row * stride + gi * group + k * 8, x);
+    const float absmax = group_max(absmax8(x), wpr);
+    const float scale = absmax / 8.0f;
+    const float inv = 1.0f / fmaxf(scale, kEps);
+    if (rl < kI4Rows) {
+      words[k * (kI4Rows + 1) + rl] = q_int4_word(x, inv);
+      if (k == 0) scale_s[rl] = scale;
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < wpr * kI4Rows; idx += kT) {
+    const int kk = idx / kI4Rows, rl = idx % kI4Rows;
+    if (r0 + rl < rows)
+      qweight[(gi * wpr + kk) * rows + r0 + rl] = (int32_t)words[kk * (kI4Rows + 1) + rl];
+  }
+  if (threadIdx.x < kI4Rows && r0 + threadIdx.x < rows)
+    store_scale(scales, sdt, gi * rows + r0 + threadIdx.x, scale_s[threadIdx.x]);
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(kT)
+dequant_int4_kernel(const int32_t* __restrict__ qweight, const void* __restrict__ scales,
+                    int sdt, int64_t rows, int group, void* __restrict__ out,
+                    int64_t ostride) {
+  extern __shared__ uint32_t i4_lds[];
+  const int wpr = group >> 3;
+  uint32_t* words = i4_lds;
+  float* scale_s = reinterpret_cast<float*>(words + wpr * (kI4Rows + 1));
+  const int64_t r0 = (int64_t)blockIdx.x * kI4Rows;
+  const int64_t gi = blockIdx.y;
+  for (int idx = threadIdx.x; idx < wpr * kI4Rows; idx += kT) {
+    const int kk = idx / kI4Rows, rl = idx % kI4Rows;
+    words[kk * (kI4Rows + 1) + rl] =
+        (r0 + rl < rows) ? (uint32_t)qweight[(gi * wpr + kk) * rows + r0 + rl] : 0u;
+  }
+  if (threadIdx.x < kI4Rows)
+    scale_s[threadIdx.x] = (r0 + threadIdx.x < rows)
+                               ? load_scale(scales, sdt, gi * rows + r0 + threadIdx.x)
+                               : 0.0f;
+  __syncthreads();
+  const int rows_per_pass = kT / wpr;
+  const int k = threadIdx.x % wpr;
+  for (int pr = 0; pr < kI4Rows; pr += rows_per_pass) {
+    const int rl = pr + threadIdx.x / wpr;
+    const int64_t row = r0 + rl;
+    if (rl >= kI4Rows || row >= rows) continue;
+    const uint32_t w = words[k * (kI4Rows + 1) + rl];
+    const float s = scale_s[rl];
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = (float)((int32_t)((w >> (4 * i)) & 0xFu) - 8) * s;
+    store8<OUT>(out, row * ostride + gi * group + k * 8, y);
+  }
+}
+
+// One lane per (row, group): any group size, any alignment.
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+quant_int4_generic(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
+                   int64_t group, int32_t* __restrict__ qweight, void* __restrict__ scales,
+                   int sdt) {
+  const int64_t ng = cols / group;
+  const int64_t t = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (t >= rows * ng) return;
+  const int64_t gi = t / rows, row = t - gi * rows;  // consecutive lanes -> consecutive rows
+  const int64_t base = row * stride + gi * group;
+  float a = 0.0f;
+  for (int64_t c = 0; c < group; ++c) a = fmaxf(a, fabsf(load1<SRC>(src, base + c)));
+  const float scale = a / 8.0f;
+  const float inv = 1.0f / fmaxf(scale, kEps);
+  store_scale(scales, sdt, gi * rows + row, scale);
+  for (int64_t k = 0; k < group / 8; ++k) {
+    float x[8];
+    for (int i = 0; i < 8; ++i) x[i] = load1<SRC>(src, base + k * 8 + i);
+    qweight[(gi * (group / 8) + k) * rows + row] = (int32_t)q_int4_word(x, inv);
+  }
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(kT)
+dequant_int4_generic(const int32_t* __restrict__ qweight, const void* __restrict__ scales,
+                     int sdt, int64_t rows, int64_t cols, int64_t group,
+                     void* __restrict__ out, int64_t ostride) {
+  const int64_t t = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (t >= rows * (cols / 8)) return;
+  const int64_t kw = t / rows, row = t - kw * rows;
+  const uint32_t w = (uint32_t)qweight[kw * rows + row];
+  const float s = load_scale(scales, sdt, ((kw * 8) / group) * rows + row);
+  for (int i = 0; i < 8; ++i)
+    store1<OUT>(out, row * ostride + kw * 8 + i,
+                (float)((int32_t)((w >> (4 * i)) & 0xFu) - 8) * s);
+}
+
+// -------------------------------------------------------------------- NF4
+
+__constant__ float kNf4Lut[16] = {
+    -1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+    -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f,
+    0.07958029955625534f, 0.16093020141124725f, 0.24611230194568634f,
+    0.33791524171829224f, 0.44070982933044434f, 0.5626170039176941f,
+    0.7229568362236023f, 1.0f};
+
+// Decision thresholds of the nearest-codebook search: the code of a normalised
+// value n is the number of thresholds t_i with n >= t_i.  t_i is the smallest
+// fp32 for which fl(|n - L[i+1]|) < fl(|n - L[i]|), found by bisection over
+// the fp32 bit patterns, so the count equals the first-minimum argmin over the
+// fp32 distances for every input (the neighbours are the only candidates: the
+// codebook spacing is >= 0.079, rounding error of a distance <= 6e-8).
+#define NF4_T(i) __uint_as_float(kNf4T[i])
+__device__ __forceinline__ uint32_t nf4_code(float n) {
+  constexpr uint32_t kNf4T[15] = {
+      0xbf591cd8u, 0xbf1c5270u, 0xbeeb847fu, 0xbeadea76u, 0xbe703cecu,
+      0xbe0d38bbu, 0xbd3a7870u, 0x3d22fb00u, 0x3df64863u, 0x3e5067e1u,
+      0x3e9582d5u, 0x3ec753fau, 0x3f006d04u, 0x3f248db0u, 0x3f5c89dau};
+  // four-level decision tree over the sorted thresholds
+  const bool b3 = n >= NF4_T(7);
+  const bool b2 = n >= (b3 ? NF4_T(11) : NF4_T(3));
+  const bool b1 = n >= (b3 ? (b2 ? NF4_T(13) : NF4_T(9)) : (b2 ? NF4_T(5) : NF4_T(1)));
+  const float t0 = b3 ? (b2 ? (b1 ? NF4_T(14) : NF4_T(12)) : (b1 ? NF4_T(10) : NF4_T(8)))
+                      : (b2 ? (b1 ? NF4_T(6) : NF4_T(4)) : (b1 ? NF4_T(2) : NF4_T(0)));
+  const bool b0 = n >= t0;
+  return ((uint32_t)b3 << 3) | ((uint32_t)b2 << 2) | ((uint32_t)b1 << 1) | (uint32_t)b0;
+}
+#undef NF4_T
+
+__device__ __forceinline__ uint32_t nf4_pack8(const float (&x)[8], float inv) {
+  uint32_t w = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t hi = nf4_code(x[2 * j] * inv), lo = nf4_code(x[2 * j + 1] * inv);
+    w |= ((hi << 4) | lo) << (8 * j);
+  }
+  return w;
+}
+
+// Flat over octets; lpg = block/8 lanes share a block (power of two <= 64).
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+quant_nf4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
+                 int lpg, uint32_t* __restrict__ packed, float* __restrict__ absmax_out) {
+  const int64_t opr = cols >> 3;
+  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
+  const bool live = o < rows * opr;
+  float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (live) {
+    const int64_t row = o / opr, c8 = o - row * opr;
+    load8<SRC>(src, row * stride + c8 * 8, x);
+  }
+  const float absmax = group_max(absmax8(x), lpg);
+  const float inv = 1.0f / fmaxf(absmax, kEps);
+  if (!live) return;
+  packed[o] = nf4_pack8(x, inv);
+  if ((threadIdx.x & (lpg - 1)) == 0) absmax_out[o / lpg] = absmax;
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(kT)
+dequant_nf4_kernel(const uint32_t* __restrict__ packed, const float* __restrict__ absmax,
+                   int64_t rows, int64_t cols, int lpg, void* __restrict__ out,
+                   int64_t ostride) {
+  __shared__ float lut[16];
+  if (threadIdx.x < 16) lut[threadIdx.x] = kNf4Lut[threadIdx.x];
+  __syncthreads();
+  const int64_t opr = cols >> 3;
+  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (o >= rows * opr) return;
+  const int64_t row = o / opr, c8 = o - row * opr;
+  const uint32_t w = packed[o];
+  const float s = absmax[o / lpg];
+  float y[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t b = (w >> (8 * j)) & 0xFFu;
+    y[2 * j] = lut[b >> 4] * s;
+    y[2 * j + 1] = lut[b & 0xFu] * s;
+  }
+  store8<OUT>(out, row * ostride + c8 * 8, y);
+}
+
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+quant_nf4_generic(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
+                  int64_t block, uint8_t* __restrict__ packed, float* __restrict__ absmax_out) {
+  const int64_t ng = cols / block;
+  const int64_t t = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (t >= rows * ng) return;
+  const int64_t row = t / ng, gi = t - row * ng;
+  const int64_t base = row * stride + gi * block;
+  float a = 0.0f;
+  for (int64_t c = 0; c < block; ++c) a = fmaxf(a, fabsf(load1<SRC>(src, base + c)));
+  const float inv = 1.0f / fmaxf(a, kEps);
+  absmax_out[t] = a;
+  for (int64_t c = 0; c < block; c += 2) {
+    const uint32_t hi = nf4_code(load1<SRC>(src, base + c) * inv);
+    const uint32_t lo = nf4_code(load1<SRC>(src, base + c + 1) * inv);
+    packed[row * (cols / 2) + (gi * block + c) / 2] = (uint8_t)((hi << 4) | lo);
+  }
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(kT)
+dequant_nf4_generic(const uint8_t* __restrict__ packed, const float* __restrict__ absmax,
+                    int64_t rows, int64_t cols, int64_t block, void* __restrict__ out,
+                    int64_t ostride) {
+  const int64_t t = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (t >= rows * (cols / 2)) return;
+  const int64_t row = t / (cols / 2), cb = t - row * (cols / 2);
+  const uint32_t b = packed[t];
+  const float s = absmax[row * (cols / block) + (cb * 2) / block];
+  store1<OUT>(out, row * ostride + cb * 2, kNf4Lut[b >> 4] * s);
+  store1<OUT>(out, row * ostride + cb * 2 + 1, kNf4Lut[b & 0xFu] * s);
+}
+
+// ------------------------------------------------------------------ NVFP4
+
+// fp32 -> float8_e4m3fn bits: round to nearest even, subnormal step 2^-9,
+// everything at or above 480 (and NaN) -> 0x7F.
+__device__ __forceinline__ uint32_t f32_to_e4m3fn_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  uint32_t a = u & 0x7FFFFFFFu;
+  uint32_t r;
+  if (a >= 0x43F00000u) {
+    r = 0x7Fu;
+  } else if (a < 0x3C800000u) {
+    r = (uint32_t)__builtin_rintf(__uint_as_float(a) * 512.0f);
+  } else {
+    const uint32_t odd = (a >> 20) & 1u;
+    a += ((uint32_t)(7 - 127) << 23) + 0x7FFFFu;
+    a += odd;
+    r = (a >> 20) & 0xFFu;
+  }
+  return sign | r;
+}
+
+__device__ __forceinline__ float e4m3fn_bits_to_f32(uint32_t b) {
+  const uint32_t sign = (b & 0x80u) << 24;
+  const uint32_t e = (b >> 3) & 0xFu, m = b & 7u;
+  uint32_t mag;
+  if (e == 0xFu && m == 7u) mag = 0x7FC00000u;
+  else if (e == 0) mag = __float_as_uint((float)m * (1.0f / 512.0f));
+  else mag = ((e + 120u) << 23) | (m << 20);
+  return __uint_as_float(sign | mag);
+}
+
+// e2m1 code, round to nearest even on the magnitude grid {0,.5,1,1.5,2,3,4,6},
+// saturating; bit 3 is the IEEE sign bit (so -0 encodes as 8).
+__device__ __forceinline__ uint32_t e2m1_code(float x) {
+  const float ax = fabsf(x);
+  const uint32_t pos = (uint32_t)(ax > 0.25f) + (uint32_t)(ax >= 0.75f) +
+                       (uint32_t)(ax > 1.25f) + (uint32_t)(ax >= 1.75f) +
+                       (uint32_t)(ax > 2.5f) + (uint32_t)(ax >= 3.5f) +
+                       (uint32_t)(ax > 5.0f);
+  return pos | ((__float_as_uint(x) >> 31) << 3);
+}
+
+__device__ __forceinline__ float e2m1_value(uint32_t code) {
+  const uint32_t pos = code & 7u;
+  uint32_t mag = ((126u + (pos >> 1)) << 23) | ((pos & 1u) << 22);
+  if (pos == 1u) mag = 126u << 23;  // 0.5: the only subnormal of the format
+  if (pos == 0u) mag = 0u;
+  return __uint_as_float(((code & 8u) << 28) | mag);
+}
+
+struct AmaxWorkspace {  // same footprint as the norm workspace
+  unsigned int ticket;
+  unsigned int pad[15];
+  float partial[1024];
+};
+
+// Tensor-wide max |x| -> global scale = max(amax, 1e-12) / (448 * 6).
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+nvfp4_global_scale_kernel(const void* __restrict__ src, int64_t stride, int64_t rows,
+                          int64_t cols, int vec, float* __restrict__ gs_out,
+                          AmaxWorkspace* __restrict__ ws) {
+  __shared__ float lds[kT / kWave];
+  __shared__ bool is_last;
+  float a = 0.0f;
+  const int64_t step = (int64_t)gridDim.x * kT;
+  if (vec) {
+    const int64_t opr = cols >> 3, total = rows * opr;
+    for (int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x; o < total; o += step) {
+      const int64_t row = o / opr, c8 = o - row * opr;
+      float x[8];
+      load8<SRC>(src, row * stride + c8 * 8, x);
+      a = fmaxf(a, absmax8(x));
+    }
+  } else {
+    const int64_t total = rows * cols;
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < total; i += step) {
+      const int64_t row = i / cols, c = i - row * cols;
+      a = fmaxf(a, fabsf(load1<SRC>(src, row * stride + c)));
+    }
+  }
+  const float m = block_max(a, lds);
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(&ws->partial[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();
+    is_last = (atomicAdd(&ws->ticket, 1u) == gridDim.x - 1);
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  float t = 0.0f;
+  for (unsigned int b = threadIdx.x; b < gridDim.x; b += kT)
+    t = fmaxf(t, __hip_atomic_load(&ws->partial[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  t = block_max(t, lds);
+  if (threadIdx.x == 0) {
+    *gs_out = fmaxf(t, kEps) / (448.0f * 6.0f);
+    __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+__device__ __forceinline__ uint32_t nvfp4_pack8(const float (&x)[8], float inv_eff) {
+  uint32_t w = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t lo = e2m1_code(x[2 * j] * inv_eff), hi = e2m1_code(x[2 * j + 1] * inv_eff);
+    w |= ((hi << 4) | lo) << (8 * j);
+  }
+  return w;
+}
+
+// block scale of a 16-element block from its amax
+__device__ __forceinline__ uint32_t nvfp4_block_scale(float amax, float inv_global) {
+  const float bs32 = fmaxf(amax, kEps) / 6.0f;
+  return f32_to_e4m3fn_bits(bs32 * inv_global);
+}
+
+// Flat over octets, two lanes per 16-element block.
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+quant_nvfp4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
+                   uint32_t* __restrict__ packed, uint8_t* __restrict__ scale8,
+                   const float* __restrict__ gs_ptr) {
+  const int64_t opr = cols >> 3, total = rows * opr;
+  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
+  const bool live = o < total;
+  float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (live) {
+    const int64_t row = o / opr, c8 = o - row * opr;
+    load8<SRC>(src, row * stride + c8 * 8, x);
+  }
+  const float gs = *gs_ptr;
+  const float inv_global = 1.0f / gs;
+  const float amax = group_max(absmax8(x), 2);
+  const uint32_t s8 = nvfp4_block_scale(amax, inv_global);
+  const float eff = e4m3fn_bits_to_f32(s8) * gs;
+  const float inv_eff = 1.0f / fmaxf(eff, kEps);
+  // gather the scales of the 4 blocks covered by 8 consecutive lanes
+  const int lane = threadIdx.x & (kWave - 1), base = lane & ~7;
+  const uint32_t s4 = __shfl(s8, base, kWave) | (__shfl(s8, base + 2, kWave) << 8) |
+                      (__shfl(s8, base + 4, kWave) << 16) | (__shfl(s8, base + 6, kWave) << 24);
+  if (!live) return;
+  packed[o] = nvfp4_pack8(x, inv_eff);
+  const int64_t o_base = o - (lane & 7);
+  if (o_base + 8 <= total) {
+    if ((lane & 7) == 0) *reinterpret_cast<uint32_t*>(scale8 + (o_base >> 1)) = s4;
+  } else if ((lane & 1) == 0) {
+    scale8[o >> 1] = (uint8_t)s8;
+  }
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(kT)
+dequant_nvfp4_kernel(const uint32_t* __restrict__ packed, const uint8_t* __restrict__ scale8,
+                     const float* __restrict__ gs_ptr, int64_t rows, int64_t cols,
+                     void* __restrict__ out, int64_t ostride) {
+  const int64_t opr = cols >> 3;
+  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (o >= rows * opr) return;
+  const int64_t row = o / opr, c8 = o - row * opr;
+  const uint32_t w = packed[o];
+  const float eff = e4m3fn_bits_to_f32(scale8[o >> 1]) * (*gs_ptr);
+  float y[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t b = (w >> (8 * j)) & 0xFFu;
+    y[2 * j] = e2m1_value(b & 0xFu) * eff;
+    y[2 * j + 1] = e2m1_value(b >> 4) * eff;
+  }
+  store8<OUT>(out, row * ostride + c8 * 8, y);
+}
+
+// One lane per 16-element block: any alignment.
+template <int SRC>
+__global__ void __launch_bounds__(kT)
+quant_nvfp4_generic(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
+                    uint8_t* __restrict__ packed, uint8_t* __restrict__ scale8,
+                    const float* __restrict__ gs_ptr) {
+  const int64_t ng = cols / 16;
+  const int64_t t = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (t >= rows * ng) return;
+  const int64_t row = t / ng, gi = t - row * ng;
+  const int64_t base = row * stride + gi * 16;
+  const float gs = *gs_ptr;
+  float a = 0.0f;
+  for (int c = 0; c < 16; ++c) a = fmaxf(a, fabsf(load1<SRC>(src, base + c)));
+  const uint32_t s8 = nvfp4_block_scale(a, 1.0f / gs);
+  scale8[t] = (uint8_t)s8;
+  const float inv_eff = 1.0f / fmaxf(e4m3fn_bits_to_f32(s8) * gs, kEps);
+  for (int c = 0; c < 16; c += 2) {
+    const uint32_t lo = e2m1_code(load1<SRC>(src, base + c) * inv_eff);
+    const uint32_t hi = e2m1_code(load1<SRC>(src, base + c + 1) * inv_eff);
+    packed[row * (cols / 2) + (gi * 16 + c) / 2] = (uint8_t)((hi << 4) | lo);
+  }
+}
+
+template <int OUT>
+__global__ void __launch_bounds__(kT)
+dequant_nvfp4_generic(const uint8_t* __restrict__ packed, const uint8_t* __restrict__ scale8,
+                      const float* __restrict__ gs_ptr, int64_t rows, int64_t cols,
+                      void* __restrict__ out, int64_t ostride) {
+  const int64_t t = (int64_t)blockIdx.x * kT + threadIdx.x;
+  if (t >= rows * (cols / 2)) return;
+  const int64_t row = t / (cols / 2), cb = t - row * (cols / 2);
+  const uint32_t b = packed[t];
+  const float eff = e4m3fn_bits_to_f32(scale8[row * (cols / 16) + cb / 8]) * (*gs_ptr);
+  store1<OUT>(out, row * ostride + cb * 2, e2m1_value(b & 0xFu) * eff);
+  store1<OUT>(out, row * ostride + cb * 2 + 1, e2m1_value(b >> 4) * eff);
+}
+
+// ------------------------------------------------------------ host helpers
+
+inline bool valid_dt(int dt) { return dt == OA_F32 || dt == OA_BF16 || dt == OA_F16; }
+inline int64_t esize(int dt) { return dt == OA_F32 ? 4 : 2; }
+inline bool pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+inline unsigned blocks_for(int64_t work) { return (unsigned)((work + kT - 1) / kT); }
+
+// fast path: rows of 8-element octets that all start on 16-byte boundaries
+inline bool rows_vec(const void* p, int dt, int64_t stride, int64_t cols) {
+  return cols % 8 == 0 && aligned_to(p, 16) && (stride * esize(dt)) % 16 == 0;
+}
+
+#define OA_DISPATCH_DT(dt, CALL)                      \
+  switch (dt) {                                       \
+    case OA_F32: { constexpr int DT = OA_F32; CALL; break; }   \
+    case OA_BF16: { constexpr int DT = OA_BF16; CALL; break; } \
+    default: { constexpr int DT = OA_F16; CALL; break; }       \
+  }
+
+int check_matrix(const void* m, int dt, int64_t stride, int64_t rows, int64_t cols) {
+  if (!valid_dt(dt) || rows < 0 || cols < 0 || stride < cols) return OA_EINVAL;
+  if (rows * cols > 0 && !m) return OA_EINVAL;
+  if (!aligned_to(m, (uintptr_t)esize(dt))) return OA_EALIGN;
+  if (rows > 0x7FFFFFFFll || rows * cols / 8 / kT > 0x7FFFFFFFll) return OA_ERANGE;
+  return 0;
+}
+
+}  // namespace
+}  // namespace oa
+
+using namespace oa;
+
+extern "C" int oa_quant_int8(const void* src, int src_dtype, int64_t src_row_stride,
+                             int64_t rows, int64_t cols, void* q, void* scales,
+                             int scale_dtype, void* stream) {
+  int rc = check_matrix(src, src_dtype, src_row_stride, rows, cols);
+  if (rc) return rc;
+  if (!valid_dt(scale_dtype)) return OA_EINVAL;
+  if (rows == 0) return 0;
+  if (!q && cols > 0) return OA_EINVAL;
+  if (!scales) return OA_EINVAL;
+  if (!aligned_to(scales, (uintptr_t)esize(scale_dtype))) return OA_EALIGN;
+  const int vec = rows_vec(src, src_dtype, src_row_stride, cols) && aligned_to(q, 8);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  OA_DISPATCH_DT(src_dtype,
+                 hipLaunchKernelGGL(quant_int8_kernel<DT>, dim3((unsigned)rows), dim3(kT), 0, s,
+                                    src, src_row_stride, cols, static_cast<int8_t*>(q), scales,
+                                    scale_dtype, vec));
+  return launch_status();
+}
+
+extern "C" int oa_dequant_int8(const void* q, const void* scales, int scale_dtype,
+                               int64_t rows, int64_t cols, void* out, int out_dtype,
+                               int64_t out_row_stride, void* stream) {
+  int rc = check_matrix(out, out_dtype, out_row_stride, rows, cols);
+  if (rc) return rc;
+  if (!valid_dt(scale_dtype)) return OA_EINVAL;
+  if (rows * cols == 0) return 0;
+  if (!q || !scales) return OA_EINVAL;
+  if (!aligned_to(scales, (uintptr_t)esize(scale_dtype))) return OA_EALIGN;
+  const int vec = rows_vec(out, out_dtype, out_row_stride, cols) && aligned_to(q, 8);
+  const int64_t work = vec ? rows * (cols / 8) : rows * cols;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  OA_DISPATCH_DT(out_dtype,
+                 hipLaunchKernelGGL(dequant_int8_kernel<DT>, dim3(blocks_for(work)), dim3(kT), 0,
+                                    s, static_cast<const int8_t*>(q), scales, scale_dtype, rows,
+                                    cols, out, out_row_stride, vec));
+  return launch_status();
+}
+
+extern "C" int oa_quant_int4(const void* src, int src_dtype, int64_t src_row_stride,
+                             int64_t rows, int64_t cols, int64_t group, void* qweight,
+                             void* scales, int scale_dtype, void* stream) {
+  int rc = check_matrix(src, src_dtype, src_row_stride, rows, cols);
+  if (rc) return rc;
+  if (!valid_dt(scale_dtype) || group <= 0 || group % 8 != 0 || cols % group != 0)
+    return OA_EINVAL;
+  if (rows * cols == 0) return 0;
+  if (!qweight || !scales) return OA_EINVAL;
+  if (!aligned_to(qweight, 4) || !aligned_to(scales, (uintptr_t)esize(scale_dtype)))
+    return OA_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t ng = cols / group;
+  const bool fast = rows_vec(src, src_dtype, src_row_stride, cols) && pow2(group) &&
+                    group <= 512 && ng <= 65535;
+  if (fast) {
+    const int wpr = (int)(group / 8);
+    const size_t lds = (size_t)wpr * (kI4Rows + 1) * 4 + kI4Rows * 4;
+    const dim3 grid((unsigned)((rows + kI4Rows - 1) / kI4Rows), (unsigned)ng);
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL(quant_int4_kernel<DT>, grid, dim3(kT), lds, s, src,
+                                      src_row_stride, rows, (int)group,
+                                      static_cast<int32_t*>(qweight), scales, scale_dtype));
+  } else {
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL(quant_int4_generic<DT>, dim3(blocks_for(rows * ng)),
+                                      dim3(kT), 0, s, src, src_row_stride, rows, cols, group,
+                                      static_cast<int32_t*>(qweight), scales, scale_dtype));
+  }
+  return launch_status();
+}
+
+extern "C" int oa_dequant_int4(const void* qweight, const void* scales, int scale_dtype,
+                               int64_t rows, int64_t cols, int64_t group, void* out,
+                               int out_dtype, int64_t out_row_stride, void* stream) {
+  int rc = check_matrix(out, out_dtype, out_row_stride, rows, cols);
+  if (rc) return rc;
+  if (!valid_dt(scale_dtype) || group <= 0 || group % 8 != 0 || cols % group != 0)
+    return OA_EINVAL;
+  if (rows * cols == 0) return 0;
+  if (!qweight || !scales) return OA_EINVAL;
+  if (!aligned_to(qweight, 4) || !aligned_to(scales, (uintptr_t)esize(scale_dtype)))
+    return OA_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t ng = cols / group;
+  const bool fast = rows_vec(out, out_dtype, out_row_stride, cols) && pow2(group) &&
+                    group <= 512 && ng <= 65535;
+  if (fast) {
+    const int wpr = (int)(group / 8);
+    const size_t lds = (size_t)wpr * (kI4Rows + 1) * 4 + kI4Rows * 4;
+    const dim3 grid((unsigned)((rows + kI4Rows - 1) / kI4Rows), (unsigned)ng);
+    OA_DISPATCH_DT(out_dtype,
+                   hipLaunchKernelGGL(dequant_int4_kernel<DT>, grid, dim3(kT), lds, s,
+                                      static_cast<const int32_t*>(qweight), scales, scale_dtype,
+                                      rows, (int)group, out, out_row_stride));
+  } else {
+    OA_DISPATCH_DT(out_dtype,
+                   hipLaunchKernelGGL(dequant_int4_generic<DT>,
+                                      dim3(blocks_for(rows * (cols / 8))), dim3(kT), 0, s,
+                                      static_cast<const int32_t*>(qweight), scales, scale_dtype,
+                                      rows, cols, group, out, out_row_stride));
+  }
+  return launch_status();
+}
+
+extern "C" int oa_quant_nf4(const void* src, int src_dtype, int64_t src_row_stride,
+                            int64_t rows, int64_t cols, int64_t block, void* packed,
+                            void* absmax, void* stream) {
+  int rc = check_matrix(src, src_dtype, src_row_stride, rows, cols);
+  if (rc) return rc;
+  if (block <= 0 || block % 2 != 0 || cols % block != 0) return OA_EINVAL;
+  if (rows * cols == 0) return 0;
+  if (!packed || !absmax) return OA_EINVAL;
+  if (!aligned_to(absmax, 4)) return OA_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool fast = rows_vec(src, src_dtype, src_row_stride, cols) && block % 8 == 0 &&
+                    pow2(block / 8) && block <= 512 && aligned_to(packed, 4);
+  if (fast) {
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL(quant_nf4_kernel<DT>, dim3(blocks_for(rows * (cols / 8))),
+                                      dim3(kT), 0, s, src, src_row_stride, rows, cols,
+                                      (int)(block / 8), static_cast<uint32_t*>(packed),
+                                      static_cast<float*>(absmax)));
+  } else {
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL(quant_nf4_generic<DT>,
+                                      dim3(blocks_for(rows * (cols / block))), dim3(kT), 0, s,
+                                      src, src_row_stride, rows, cols, block,
+                                      static_cast<uint8_t*>(packed), static_cast<float*>(absmax)));
+  }
+  return launch_status();
+}
+
+extern "C" int oa_dequant_nf4(const void* packed, const void* absmax, int64_t rows,
+                              int64_t cols, int64_t block, void* out, int out_dtype,
+                              int64_t out_row_stride, void* stream) {
+  int rc = check_matrix(out, out_dtype, out_row_stride, rows, cols);
+  if (rc) return rc;
+  if (block <= 0 || block % 2 != 0 || cols % block != 0) return OA_EINVAL;
+  if (rows * cols == 0) return 0;
+  if (!packed || !absmax) return OA_EINVAL;
+  if (!aligned_to(absmax, 4)) return OA_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool fast = rows_vec(out, out_dtype, out_row_stride, cols) && block % 8 == 0 &&
+                    pow2(block / 8) && block <= 512 && aligned_to(packed, 4);
+  if (fast) {
+    OA_DISPATCH_DT(out_dtype,
+                   hipLaunchKernelGGL(dequant_nf4_kernel<DT>, dim3(blocks_for(rows * (cols / 8))),
+                                      dim3(kT), 0, s, static_cast<const uint32_t*>(packed),
+                                      static_cast<const float*>(absmax), rows, cols,
+                                      (int)(block / 8), out, out_row_stride));
+  } else {
+    OA_DISPATCH_DT(out_dtype,
+                   hipLaunchKernelGGL(dequant_nf4_generic<DT>,
+                                      dim3(blocks_for(rows * (cols / 2))), dim3(kT), 0, s,
+                                      static_cast<const uint8_t*>(packed),
+                                      static_cast<const float*>(absmax), rows, cols, block, out,
+                                      out_row_stride));
+  }
+  return launch_status();
+}
+
+extern "C" int oa_quant_nvfp4(const void* src, int src_dtype, int64_t src_row_stride,
+                              int64_t rows, int64_t cols, void* packed, void* block_scale,
+                              void* global_scale, void* workspace, void* stream) {
+  int rc = check_matrix(src, src_dtype, src_row_stride, rows, cols);
+  if (rc) return rc;
+  if (cols % 16 != 0 || !global_scale || !workspace) return OA_EINVAL;
+  if (!aligned_to(global_scale, 4) || !aligned_to(workspace, 64)) return OA_EALIGN;
+  if (rows * cols > 0 && (!packed || !block_scale)) return OA_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int vec = rows_vec(src, src_dtype, src_row_stride, cols);
+  const int64_t work = vec ? rows * (cols / 8) : rows * cols;
+  int64_t rblocks = (work + (int64_t)kT * 8 - 1) / ((int64_t)kT * 8);
+  if (rblocks < 1) rblocks = 1;
+  if (rblocks > 1024) rblocks = 1024;
+  OA_DISPATCH_DT(src_dtype,
+                 hipLaunchKernelGGL(nvfp4_global_scale_kernel<DT>, dim3((unsigned)rblocks),
+                                    dim3(kT), 0, s, src, src_row_stride, rows, cols, vec,
+                                    static_cast<float*>(global_scale),
+                                    static_cast<AmaxWorkspace*>(workspace)));
+  rc = launch_status();
+  if (rc || rows * cols == 0) return rc;
+  if (vec && aligned_to(packed, 4) && aligned_to(block_scale, 4)) {
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL(quant_nvfp4_kernel<DT>, dim3(blocks_for(rows * (cols / 8))),
+                                      dim3(kT), 0, s, src, src_row_stride, rows, cols,
+                                      static_cast<uint32_t*>(packed),
+                                      static_cast<uint8_t*>(block_scale),
+                                      static_cast<const float*>(global_scale)));
+  } else {
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL(quant_nvfp4_generic<DT>,
+                                      dim3(blocks_for(rows * (cols / 16))), dim3(kT), 0, s, src,
+                                      src_row_stride, rows, cols, static_cast<uint8_t*>(packed),
+                                      static_cast<uint8_t*>(block_scale),
+                                      static_cast<const float*>(global_scale)));
+  }
+  return launch_status();
+}
+
+extern "C" int oa_dequant_nvfp4(const void* packed, const void* block_scale,
+                                const void* global_scale, int64_t rows, int64_t cols,
+                                void* out, int out_dtype, int64_t out_row_stride,
+                                void* stream) {
+  int rc = check_matrix(out, out_dtype, out_row_stride, rows, cols);
+  if (rc) return rc;
+  if (cols % 16 != 0) return OA_EINVAL;
+  if (rows * cols == 0) return 0;
+  if (!packed || !block_scale || !global_scale) return OA_EINVAL;
+  if (!aligned_to(global_scale, 4)) return OA_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (rows_vec(out, out_dtype, out_row_stride, cols) && aligned_to(packed, 4)) {
+    OA_DISPATCH_DT(out_dtype,
+                   hipLaunchKernelGGL(dequant_nvfp4_kernel<DT>,
+                                      dim3(blocks_for(rows * (cols / 8))), dim3(kT), 0, s,
+                                      static_cast<const uint32_t*>(packed),
+                                      static_cast<const uint8_t*>(block_scale),
+                                      static_cast<const float*>(global_scale), rows, cols, out,
+                                      out_row_stride));
+  } else {
+    OA_DISPATCH_DT(out_dtype,
+                   hipLaunchKernelGGL(dequant_nvfp4_generic<DT>,
+                                      dim3(blocks_for(rows * (cols / 2))), dim3(kT), 0, s,
+                                      static_cast<const uint8_t*>(packed),
+                                      static_cast<const uint8_t*>(block_scale),
+                                      static_cast<const float*>(global_scale), rows, cols, out,
+                                      out_row_stride));
+  }
+  return launch_status();
+}

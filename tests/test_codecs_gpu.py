@@ -1,0 +1,233 @@
+"""GPU parity of the eight codec kernels against the C oracle: BIT-EXACT on the
+packed codes, the scales and the dequantised values.
+
+Shapes follow the reference's own parity tests (tests/test_int8.py:70-84 and
+the other three files): seeded ``randn * 0.05`` in bf16 / fp16, plus fp32
+masters, misaligned row counts, column counts off the 8-element fast path,
+strided and unaligned sources, and BASELINE config 3 (4096 x 14336 with 1 %
+outliers x10).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DT = {torch.float32: "float32", torch.bfloat16: "bfloat16", torch.float16: "float16"}
+
+
+def _weight(rows, cols, dtype, seed=0, outliers=False):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(rows, cols, generator=g) * (0.02 if outliers else 0.05)
+    if outliers:
+        mask = torch.rand(rows, cols, generator=g) < 0.01
+        w = torch.where(mask, w * 10, w)
+    return w.to(dtype)
+
+
+def _np_bits(t):
+    """float tensor -> numpy array of raw bits (uint16 for 16-bit, uint32 for fp32)."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.float32:
+        return t.numpy().view(np.uint32)
+    return t.view(torch.int16).numpy().view(np.uint16)
+
+
+def _oracle_out_bits(a, out_dtype):
+    return a.view(np.uint32) if out_dtype == torch.float32 else a
+
+
+def _cast_scales(s_f32, dtype):
+    """fp32 oracle scales -> bits after torch's own cast to the scale dtype."""
+    return _np_bits(torch.from_numpy(s_f32.copy()).to(dtype))
+
+
+SHAPES = [(128, 256), (35, 256), (4096, 4096), (64, 2048)]
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES + [(64, 37), (3, 8), (1, 1)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_int8(oracle, rows, cols, dtype):
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    w = _weight(rows, cols, dtype)
+    sdt = torch.bfloat16 if dtype == torch.float32 else dtype
+    q = torch.empty(rows, cols, dtype=torch.int8, device="cuda")
+    s = torch.empty(rows, dtype=sdt, device="cuda")
+    ops.quantize_int8_into(w.cuda(), q, s)
+    rq, rs = oracle.quant_int8(w.float().numpy())
+    assert np.array_equal(q.cpu().numpy(), rq)
+    assert np.array_equal(_np_bits(s), _cast_scales(rs, sdt))
+    for odt in (sdt, torch.float32):
+        got = ops.dequantize_int8(q, s, odt)
+        want = oracle.dequant_int8(rq, s.float().cpu().numpy(), DT[odt])
+        assert np.array_equal(_np_bits(got), _oracle_out_bits(want, odt)), odt
+
+
+@pytest.mark.parametrize("rows,cols,group", [(128, 256, 128), (35, 256, 128), (4096, 4096, 128),
+                                             (64, 2048, 64), (40, 96, 32), (8, 48, 24),
+                                             (5, 1024, 512)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_int4(oracle, rows, cols, group, dtype):
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    w = _weight(rows, cols, dtype, seed=1)
+    sdt = torch.bfloat16 if dtype == torch.float32 else dtype
+    qw = torch.empty(cols // 8, rows, dtype=torch.int32, device="cuda")
+    s = torch.empty(cols // group, rows, dtype=sdt, device="cuda")
+    ops.quantize_int4_into(w.cuda(), group, qw, s)
+    rq, rs = oracle.quant_int4(w.float().numpy(), group)
+    assert np.array_equal(qw.cpu().numpy(), rq)
+    assert np.array_equal(_np_bits(s), _cast_scales(rs, sdt))
+    for odt in (sdt, torch.float32):
+        got = ops.dequantize_int4(qw, s, group, odt)
+        want = oracle.dequant_int4(rq, s.float().cpu().numpy(), group, DT[odt])
+        assert np.array_equal(_np_bits(got), _oracle_out_bits(want, odt)), odt
+
+
+@pytest.mark.parametrize("rows,cols,block", [(128, 256, 64), (35, 256, 64), (4096, 4096, 64),
+                                             (64, 128, 32), (16, 60, 6), (7, 1024, 512)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_nf4(oracle, rows, cols, block, dtype):
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    w = _weight(rows, cols, dtype, seed=2)
+    packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    absmax = torch.empty(rows * (cols // block), dtype=torch.float32, device="cuda")
+    ops.quantize_nf4_into(w.cuda(), block, packed, absmax)
+    rp, ra = oracle.quant_nf4(w.float().numpy(), block)
+    assert np.array_equal(absmax.cpu().numpy().view(np.uint32), ra.view(np.uint32))
+    assert np.array_equal(packed.cpu().numpy(), rp)
+    for odt in (torch.bfloat16, torch.float16, torch.float32):
+        got = ops.dequantize_nf4(packed, absmax, cols, block, odt)
+        want = oracle.dequant_nf4(rp, ra, block, DT[odt])
+        assert np.array_equal(_np_bits(got), _oracle_out_bits(want, odt)), odt
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES + [(35, 16), (3, 48)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_nvfp4(oracle, rows, cols, dtype):
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    w = _weight(rows, cols, dtype, seed=3)
+    packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    s8 = torch.empty(rows, cols // 16, dtype=torch.float8_e4m3fn, device="cuda")
+    gs = torch.empty((), dtype=torch.float32, device="cuda")
+    ops.quantize_nvfp4_into(w.cuda(), packed, s8, gs)
+    rp, rs, rgs = oracle.quant_nvfp4(w.float().numpy())
+    assert gs.cpu().numpy().view(np.uint32) == np.float32(rgs).view(np.uint32)
+    assert np.array_equal(s8.view(torch.uint8).cpu().numpy(), rs)
+    assert np.array_equal(packed.cpu().numpy(), rp)
+    for odt in (torch.bfloat16, torch.float16, torch.float32):
+        got = ops.dequantize_nvfp4(packed, s8, gs, cols, odt)
+        want = oracle.dequant_nvfp4(rp, rs, rgs, DT[odt])
+        assert np.array_equal(_np_bits(got), _oracle_out_bits(want, odt)), odt
+
+
+def test_strided_and_unaligned_sources(oracle):
+    """Column slices (row stride > cols) and views starting off a 16-byte
+    boundary give the same codes as the contiguous copy."""
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    big = _weight(64, 512 + 8, torch.float32, seed=4).cuda()
+    for view in (big[:, :512], big[:, 8:520], big[:, 3:515]):
+        rows, cols = view.shape
+        ref = view.contiguous().cpu().numpy()
+        q = torch.empty(rows, cols, dtype=torch.int8, device="cuda")
+        s = torch.empty(rows, dtype=torch.bfloat16, device="cuda")
+        ops.quantize_int8_into(view, q, s)
+        assert np.array_equal(q.cpu().numpy(), oracle.quant_int8(ref)[0])
+        qw = torch.empty(cols // 8, rows, dtype=torch.int32, device="cuda")
+        s4 = torch.empty(cols // 128, rows, dtype=torch.bfloat16, device="cuda")
+        ops.quantize_int4_into(view, 128, qw, s4)
+        assert np.array_equal(qw.cpu().numpy(), oracle.quant_int4(ref, 128)[0])
+        pk = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+        am = torch.empty(rows * (cols // 64), dtype=torch.float32, device="cuda")
+        ops.quantize_nf4_into(view, 64, pk, am)
+        assert np.array_equal(pk.cpu().numpy(), oracle.quant_nf4(ref, 64)[0])
+        pk4 = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+        s8 = torch.empty(rows, cols // 16, dtype=torch.float8_e4m3fn, device="cuda")
+        gs = torch.empty((), dtype=torch.float32, device="cuda")
+        ops.quantize_nvfp4_into(view, pk4, s8, gs)
+        rp, rs, _ = oracle.quant_nvfp4(ref)
+        assert np.array_equal(pk4.cpu().numpy(), rp)
+        assert np.array_equal(s8.view(torch.uint8).cpu().numpy(), rs)
+
+
+def test_nf4_thresholds_match_brute_force(oracle):
+    """The kernel's threshold tree must equal the 16-way fp32 distance search for
+    every input: all floats within 64 ulps of each decision point, the codebook
+    itself, and a dense sweep of [-1, 1]."""
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    lut = np.array([oracle.lib().oaref_nf4_lut(i) for i in range(16)], dtype=np.float32)
+    mids = ((lut[:-1].astype(np.float64) + lut[1:]) / 2).astype(np.float32)
+    pts = [lut, np.linspace(-1, 1, 200_001, dtype=np.float32)]
+    for m in mids:
+        b = int(m.view(np.uint32))
+        pts.append(np.arange(b - 64, b + 65, dtype=np.uint32).view(np.float32))
+    x = np.concatenate(pts)
+    pad = (-len(x)) % 64
+    x = np.concatenate([x, np.zeros(pad, dtype=np.float32)])
+    # one row per 64-block whose absmax is exactly 1, so normalised == input
+    x = x.reshape(-1, 64)
+    x = np.concatenate([x, np.ones((x.shape[0], 64), dtype=np.float32)], axis=1)
+    t = torch.from_numpy(x).cuda()
+    rows, cols = t.shape
+    packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    absmax = torch.empty(rows, dtype=torch.float32, device="cuda")
+    # block = 128 covers the data half and the all-ones half: absmax == 1
+    ops.quantize_nf4_into(t, 128, packed, absmax)
+    rp, _ = oracle.quant_nf4(x, 128)
+    assert np.array_equal(packed.cpu().numpy(), rp)
+
+
+def test_config3_weight(oracle):
+    """BASELINE config 3: 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
+    x10; requantise from its fp32 master, every format, then dequantise."""
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    rows, cols = 4096, 14336
+    w = _weight(rows, cols, torch.bfloat16, seed=5, outliers=True)
+    master = w.float()
+    m_gpu = master.cuda()
+    m_np = master.numpy()
+
+    q = torch.empty(rows, cols, dtype=torch.int8, device="cuda")
+    s = torch.empty(rows, dtype=torch.bfloat16, device="cuda")
+    ops.quantize_int8_into(m_gpu, q, s)
+    rq, rs = oracle.quant_int8(m_np)
+    assert np.array_equal(q.cpu().numpy(), rq)
+    assert np.array_equal(_np_bits(s), _cast_scales(rs, torch.bfloat16))
+    assert np.array_equal(_np_bits(ops.dequantize_int8(q, s)),
+                          oracle.dequant_int8(rq, s.float().cpu().numpy(), "bfloat16"))
+
+    qw = torch.empty(cols // 8, rows, dtype=torch.int32, device="cuda")
+    s4 = torch.empty(cols // 128, rows, dtype=torch.bfloat16, device="cuda")
+    ops.quantize_int4_into(m_gpu, 128, qw, s4)
+    rq4, rs4 = oracle.quant_int4(m_np, 128)
+    assert np.array_equal(qw.cpu().numpy(), rq4)
+    assert np.array_equal(_np_bits(s4), _cast_scales(rs4, torch.bfloat16))
+    assert np.array_equal(_np_bits(ops.dequantize_int4(qw, s4, 128)),
+                          oracle.dequant_int4(rq4, s4.float().cpu().numpy(), 128, "bfloat16"))
+
+    pk = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    am = torch.empty(rows * (cols // 64), dtype=torch.float32, device="cuda")
+    ops.quantize_nf4_into(m_gpu, 64, pk, am)
+    rp, ra = oracle.quant_nf4(m_np, 64)
+    assert np.array_equal(pk.cpu().numpy(), rp)
+    assert np.array_equal(am.cpu().numpy().view(np.uint32), ra.view(np.uint32))
+    assert np.array_equal(_np_bits(ops.dequantize_nf4(pk, am, cols, 64, torch.bfloat16)),
+                          oracle.dequant_nf4(rp, ra, 64, "bfloat16"))
+
+    pk4 = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    s8 = torch.empty(rows, cols // 16, dtype=torch.float8_e4m3fn, device="cuda")
+    gs = torch.empty((), dtype=torch.float32, device="cuda")
+    ops.quantize_nvfp4_into(m_gpu, pk4, s8, gs)
+    rp4, rs8, rgs = oracle.quant_nvfp4(m_np)
+    assert gs.cpu().numpy().view(np.uint32) == np.float32(rgs).view(np.uint32)
+    assert np.array_equal(pk4.cpu().numpy(), rp4)
+    assert np.array_equal(s8.view(torch.uint8).cpu().numpy(), rs8)
+    assert np.array_equal(_np_bits(ops.dequantize_nvfp4(pk4, s8, gs, cols, torch.bfloat16)),
+                          oracle.dequant_nvfp4(rp4, rs8, rgs, "bfloat16"))
