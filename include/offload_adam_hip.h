@@ -41,6 +41,8 @@ extern "C" {
 #define OA_EALIGN   (-2) /* pointer not aligned to its element type */
 #define OA_ERANGE   (-3) /* size beyond what the entry point supports */
 #define OA_EOVERLAP (-4) /* buffers that must be distinct alias each other */
+#define OA_EOS      (-5) /* an operating-system call failed; errno is reported
+                            through the entry point's os_errno argument */
 
 /* ABI version of the loaded library (== OA_ABI_VERSION it was built with). */
 int oa_abi_version(void);
@@ -240,6 +242,39 @@ int oa_dequant_nvfp4(const void* packed, const void* block_scale,
                      const void* global_scale, int64_t rows, int64_t cols,
                      void* out, int out_dtype, int64_t out_row_stride,
                      void* stream);
+
+/* ------------------------------------------------------------------------
+ * D. Pinned host memory and host<->device streaming.
+ * ---------------------------------------------------------------------- */
+
+/* Replaces the mmap / mbind / memset / cudaHostRegister sequence of
+ * pinned_alloc._alloc (src/offload_adam/pinned_alloc.py:177-235).
+ * Allocates `bytes` rounded up to 4 KiB pages of zero-filled, page-locked host
+ * memory.  numa_node >= 0 prefers that node softly (MPOL_PREFERRED: spills to
+ * other nodes when it is full); -1 leaves placement to the HIP runtime.
+ * Returns 0 and the address in *out; OA_EOS with the OS errno in *os_errno
+ * when the memory-policy call fails; a positive hipError_t when the runtime
+ * cannot allocate or pin. */
+int oa_pinned_alloc(size_t bytes, int numa_node, void** out, int* os_errno);
+
+/* Releases memory obtained from oa_pinned_alloc (the cleanup closure of
+ * pinned_alloc.py:222-232). */
+int oa_pinned_free(void* ptr);
+
+/* Replaces pinned_alloc.gpu_numa_node (src/offload_adam/pinned_alloc.py:113-128):
+ * NUMA node of the PCI device behind HIP device `device`, -1 when the kernel
+ * reports none. */
+int oa_gpu_numa_node(int device, int* node_out);
+
+/* Asynchronous copy on `stream`; stands in for the `Tensor.to(non_blocking)` /
+ * `copy_(non_blocking)` calls of OffloadAdam._issue_h2d / _issue_d2h
+ * (src/offload_adam/offload_adam.py:347-372).  The host side must be
+ * page-locked for the copy to be asynchronous.  Ordering against other streams
+ * is the caller's job (events). */
+#define OA_COPY_H2D 0
+#define OA_COPY_D2H 1
+#define OA_COPY_D2D 2
+int oa_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream);
 
 #ifdef __cplusplus
 }

@@ -83,8 +83,17 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p],
     ),
+    "oa_pinned_alloc": (
+        c_int,
+        [c_size_t, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int)],
+    ),
+    "oa_pinned_free": (c_int, [c_void_p]),
+    "oa_gpu_numa_node": (c_int, [c_int, ctypes.POINTER(c_int)]),
+    "oa_memcpy_async": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
 }
 
+OA_EOS = -5
+OA_COPY_H2D, OA_COPY_D2H, OA_COPY_D2D = 0, 1, 2
 OA_F32, OA_BF16, OA_F16 = 0, 1, 2
 
 

@@ -15,6 +15,8 @@ extern "C" const char* oa_error_string(int code) {
       return "offload_adam_hip: size is beyond what this entry point supports";
     case OA_EOVERLAP:
       return "offload_adam_hip: buffers that must be distinct alias each other";
+    case OA_EOS:
+      return "offload_adam_hip: an operating-system call failed (see os_errno)";
     default:
       break;
   }

@@ -1,0 +1,517 @@
+"""``OffloadAdam``: Adam whose gradients and optimizer states live in pinned host
+memory and visit the GPU only for the step.
+
+Drop-in for the reference's ``offload_adam.OffloadAdam``
+(src/offload_adam/offload_adam.py:39-678): same constructor knobs, mode
+strings, ``ready_for_optimizer_step`` contract, per-parameter state layout and
+the two execution paths selected by ``max_grad_norm``:
+
+* ``max_grad_norm=None`` - the whole step of a parameter (H2D of its states,
+  fused AdamW kernel, D2H write-back) runs inside that parameter's
+  post-accumulate-grad hook on the last micro-batch, overlapping with the rest
+  of backward;
+* ``max_grad_norm=float`` - backward only accumulates gradients and records
+  per-parameter L2 norms; ``step()`` forms the global clip coefficient on the
+  GPU (no host sync) and walks the parameters, prefetching the next
+  parameter's states while the current one is updated.
+
+What runs underneath is this package's HIP library: the fused AdamW kernels
+(with the clip coefficient folded into the gradient load instead of a separate
+``grad.mul_`` pass), the norm / coefficient kernels, the pinned allocator and
+``hipMemcpyAsync`` on two side streams fenced with events.
+"""
+
+import warnings
+from ctypes import c_int, c_size_t, c_void_p
+
+import torch
+from torch.optim.optimizer import Optimizer
+
+from . import _lib, grad_clip
+from ._pretrained import stream_master_from_pretrained
+from .adam import _LOSSY_MASTER_HINT, MODE_TABLE
+from .pinned_alloc import numa_node_free_bytes, resolve_numa_target, zeros_pinned
+from .qweight.base import QWeightBase
+
+_BF16 = torch.bfloat16
+_GIB = 1024**3
+
+
+def get_leaf_modules_with_params(module):
+    """Leaf modules (no children) that directly own a trainable parameter, in
+    registration order.  Parameters held by a module that also has children are
+    not seen (same scan as the reference, offload_adam.py:28-36)."""
+    found = []
+    for child in module.children():
+        if any(True for _ in child.children()):
+            found.extend(get_leaf_modules_with_params(child))
+        elif any(p.requires_grad for p in child.parameters(recurse=False)):
+            found.append(child)
+    return found
+
+
+def _copy_async(dst, src, kind, stream):
+    """hipMemcpyAsync of a whole contiguous tensor on ``stream``."""
+    nbytes = src.numel() * src.element_size()
+    code = _lib.load().oa_memcpy_async(
+        c_void_p(dst.data_ptr()), c_void_p(src.data_ptr()), c_size_t(nbytes), c_int(kind),
+        c_void_p(stream.cuda_stream),
+    )
+    _lib.check(code, "oa_memcpy_async")
+
+
+class OffloadAdam(Optimizer):
+    """Adam with gradients and optimizer states offloaded to pinned host memory.
+
+    Args:
+        model (nn.Module): model whose leaf-module parameters are optimized.
+        lr, betas, eps, weight_decay: the usual Adam hyper-parameters
+            (defaults 1e-3, (0.9, 0.999), 1e-8, 0.01).
+        mode (str): ``'stochastic_rounding'`` (default), ``'fp32_master'``,
+            ``'fp31_master'`` or ``'fp32_master_custom_rounding'``.
+        max_grad_norm (float | None): global L2-norm clipping threshold; ``None``
+            (default) moves the step into the backward hooks.
+        numa_node (str | int | None): NUMA placement of the pinned buffers -
+            ``'auto'`` (the GPU's node), a node id, or ``None``.
+        decoupled_weight_decay (bool): AdamW-style decay. Default False.
+        inplace_param_threshold (int | None): parameters with fewer elements keep
+            gradient and states on the GPU and never cross PCIe. Default 1M;
+            ``0`` offloads everything.
+        prefetch_policy (str): ``'eager'`` (default) starts a parameter's H2D at
+            the first backward-pre hook that sees it; ``'lazy'`` waits for the
+            module that owns it first in forward order (matters for parameters
+            shared by several modules, e.g. tied embeddings).
+        verbose (int): non-zero prints the pinned / in-place byte totals.
+    """
+
+    supported_modes = {
+        mode: {
+            "step": fn,
+            "offload": {"grad": _BF16, "exp_avg": _BF16, "exp_avg_sq": _BF16, **extra},
+        }
+        for mode, (fn, extra) in MODE_TABLE.items()
+    }
+
+    _DEFAULT_INPLACE_PARAM_THRESHOLD = 1024 * 1024
+    _CLIP_PREFETCH_DEPTH = 2  # parameters whose H2D runs ahead of the step loop
+
+    def __init__(
+        self,
+        model,
+        lr=1e-3,
+        betas=(0.9, 0.999),
+        eps=1e-8,
+        weight_decay=0.01,
+        mode="stochastic_rounding",
+        max_grad_norm=None,
+        numa_node="auto",
+        decoupled_weight_decay=False,
+        inplace_param_threshold=None,
+        prefetch_policy="eager",
+        verbose=0,
+    ):
+        if prefetch_policy not in ("eager", "lazy"):
+            raise ValueError(f"prefetch_policy must be 'eager' or 'lazy' (got {prefetch_policy!r})")
+        self._prefetch_policy = prefetch_policy
+        assert mode in self.supported_modes, (
+            f"Invalid mode: {mode}, available modes: {list(self.supported_modes)}"
+        )
+        self.mode = mode
+        self.step_fn = self.supported_modes[mode]["step"]
+        self.offload_config = self.supported_modes[mode]["offload"]
+        self.offload_state_keys = list(self.offload_config)
+        self._non_grad_keys = [k for k in self.offload_state_keys if k != "grad"]
+
+        self.max_grad_norm = max_grad_norm
+        self._step_in_backward = max_grad_norm is None
+        self.decoupled_weight_decay = decoupled_weight_decay
+        self.verbose = verbose
+        self.ready_for_optimizer_step = False
+
+        modules = get_leaf_modules_with_params(model)
+        params, owners = [], {}
+        for m in modules:
+            for p in m.parameters():
+                if p.requires_grad:
+                    if id(p) not in owners:
+                        params.append(p)  # tied weights enter the optimizer once
+                    owners[id(p)] = owners.get(id(p), 0) + 1
+        shared = [p for p in params if owners[id(p)] > 1]
+        if shared and prefetch_policy == "eager":
+            warnings.warn(
+                f"OffloadAdam: {len(shared)} parameter(s) shared across multiple leaf modules "
+                f"({sum(p.numel() for p in shared):,} elements; e.g. tied embeddings). With "
+                f"prefetch_policy='eager' their non-grad states sit on GPU through the whole "
+                f"backward. Pass prefetch_policy='lazy' to defer prefetch to the input-side "
+                f"module.",
+                stacklevel=2,
+            )
+        super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
+
+        self._quant_params = {p for p in params if isinstance(p.data, QWeightBase)}
+        if self._quant_params and mode != "fp32_master":
+            raise ValueError(
+                f"QAT params require mode='fp32_master'; got {mode!r} "
+                f"({len(self._quant_params)} quant params detected)"
+            )
+        self._quant_master_warned = False
+
+        if inplace_param_threshold is None:
+            inplace_param_threshold = self._DEFAULT_INPLACE_PARAM_THRESHOLD
+        self.inplace_param_threshold = inplace_param_threshold
+        # quantised params always offload: their fp32 master belongs on the host
+        self._inplace_params = {
+            p for p in params
+            if p.numel() < inplace_param_threshold and p not in self._quant_params
+        }
+        self._offload_params = [p for p in params if p not in self._inplace_params]
+
+        self.device_states = {}
+        self.h2d_events = {}
+        self.d2h_events = {}
+        self.h2d_stream = torch.cuda.Stream()
+        self.d2h_stream = torch.cuda.Stream()
+        self._param2group = {p: g for g in self.param_groups for p in g["params"]}
+        # first module in forward order that owns each offloaded param ('lazy' policy)
+        self._prefetch_module = {}
+        for m in modules:
+            for p in m.parameters():
+                if p.requires_grad and p not in self._inplace_params:
+                    self._prefetch_module.setdefault(p, m)
+
+        # clipping: one bf16 slot per parameter, reduced by one kernel in step()
+        self._norm_slots = None
+        self._clip_coef = None
+        if max_grad_norm is not None:
+            dev = params[0].device if params else torch.device("cuda")
+            self._norm_slots = torch.zeros(max(len(params), 1), dtype=_BF16, device=dev)
+            self._clip_coef = torch.ones((), dtype=_BF16, device=dev)
+            self._total_norm = torch.zeros((), dtype=_BF16, device=dev)
+
+        self._register_hooks(modules, params)
+        self._numa_precheck(self._offload_params, numa_node)
+        self._alloc_pinned_states(self._offload_params, numa_node)
+        self._alloc_inplace_states(self._inplace_params)
+
+    # ------------------------------------------------------------------ setup
+
+    def _register_hooks(self, modules, params):
+        for module in modules:
+            if any(p.requires_grad and p not in self._inplace_params for p in module.parameters()):
+                module.register_full_backward_pre_hook(self._pre_backward_hook)
+        for index, p in enumerate(params):
+            state = self.state[p]
+            state["step"] = 0
+            if self.max_grad_norm is not None:
+                state["grad_norm"] = self._norm_slots[index]  # 0-dim view of the shared buffer
+            if p in self._inplace_params:
+                p.register_post_accumulate_grad_hook(self._inplace_grad_hook)
+            else:
+                p.register_post_accumulate_grad_hook(self._grad_hook)
+                self.device_states[p] = {}
+                state["host_grad_valid"] = False
+
+    def _estimate_pinned_bytes(self, params):
+        per_elem = sum(torch.empty(0, dtype=d).element_size() for d in self.offload_config.values())
+        return sum(p.numel() for p in params) * per_elem
+
+    def _numa_precheck(self, params, numa_node):
+        """Warn when the target NUMA node cannot hold the pinned budget: the soft
+        node preference then spills the rest to remote nodes."""
+        target = resolve_numa_target(numa_node)
+        if target is None or not params:
+            return
+        free = numa_node_free_bytes(target)
+        if free is None:
+            return
+        need = self._estimate_pinned_bytes(params)
+        world_size = getattr(self, "_world_size", 1)
+        fair_share = free // world_size
+        if need > fair_share:
+            warnings.warn(
+                f"OffloadAdam: need {need / _GIB:.1f} GB pinned on NUMA node {target} "
+                f"({world_size} rank(s) sharing) but fair share is {fair_share / _GIB:.1f} GB; "
+                f"~{(need - fair_share) / _GIB:.1f} GB will spill to remote nodes (H2D may slow "
+                f"~10-15%). Pass `numa_node=None` to let the kernel spread freely, or move GPUs "
+                f"to separate NUMA domains.",
+                stacklevel=3,
+            )
+
+    def _copy_master(self, p, tensor):
+        self.state[p]["master_params"].copy_(tensor)
+
+    def _alloc_pinned_states(self, params, numa_node):
+        total = 0
+        for p in params:
+            state = self.state[p]
+            for name, dtype in self.offload_config.items():
+                t = zeros_pinned(p.shape, dtype, numa_node=numa_node)
+                if name == "master_params":
+                    t.copy_(p.data)  # widens bf16 losslessly; dequantises a quantised weight
+                state[name] = t
+                total += t.numel() * t.element_size()
+            if p in self._quant_params and "master_params" in self.offload_config:
+                state["master_filled"] = False
+        if self.verbose > 0 and params:
+            print(f"Pinned host memory allocated: {total / _GIB:.2f} GB")
+
+    def _alloc_inplace_states(self, params):
+        """GPU-resident gradient and states of the small parameters.  The gradient
+        buffer starts at zero and is zeroed after every step, so the hook can
+        always ``add_`` into it."""
+        total = 0
+        for p in params:
+            state = self.state[p]
+            for name, dtype in self.offload_config.items():
+                t = torch.zeros_like(p, dtype=dtype)
+                if name == "master_params":
+                    t.copy_(p.data)
+                state[name] = t
+                total += t.numel() * t.element_size()
+        if self.verbose > 0 and params:
+            print(f"In-place GPU states for {len(params)} small params: {total / 1024**2:.2f} MB")
+
+    # --------------------------------------------------- transfer primitives
+    # Ordering contract, per parameter p:
+    #   H2D(p) starts after D2H(p) of the previous step and after everything the
+    #   compute stream has enqueued so far (its destination buffers come from the
+    #   compute stream's allocator pool);
+    #   the compute stream waits for H2D(p) before touching p's device states;
+    #   D2H(p) starts after everything the compute stream has enqueued so far;
+    #   a device buffer is not recycled before the D2H that reads it is done.
+
+    def _host_view(self, p, name):
+        return self.state[p][name]
+
+    def _issue_h2d(self, p, keys):
+        compute = torch.cuda.current_stream()
+        dev = self.device_states[p]
+        if p in self.d2h_events:
+            self.h2d_stream.wait_event(self.d2h_events[p])
+        self.h2d_stream.wait_stream(compute)
+        for key in keys:
+            host = self._host_view(p, key)
+            buf = torch.empty(host.shape, dtype=host.dtype, device=p.device)
+            _copy_async(buf, host, _lib.OA_COPY_H2D, self.h2d_stream)
+            dev[key] = buf
+        self.h2d_events[p] = self.h2d_stream.record_event()
+
+    def _issue_d2h(self, p, keys):
+        compute = torch.cuda.current_stream()
+        dev = self.device_states[p]
+        self.d2h_stream.wait_stream(compute)
+        for key in keys:
+            buf = dev[key]
+            _copy_async(self._host_view(p, key), buf, _lib.OA_COPY_D2H, self.d2h_stream)
+            buf.record_stream(self.d2h_stream)
+            dev[key] = None
+        self.d2h_events[p] = self.d2h_stream.record_event()
+
+    def _ensure_on_device(self, p, keys):
+        dev = self.device_states[p]
+        missing = [k for k in keys if dev.get(k) is None]
+        if missing:
+            self._issue_h2d(p, missing)
+        if p in self.h2d_events:
+            torch.cuda.current_stream().wait_event(self.h2d_events[p])
+
+    # ------------------------------------------------- per-parameter operations
+
+    def _accumulate_grad_on_device(self, p):
+        """First micro-batch of a window adopts ``p.grad`` as the device gradient;
+        later ones wait for the prefetched host gradient and add into it."""
+        dev, state = self.device_states[p], self.state[p]
+        if state["host_grad_valid"]:
+            self._ensure_on_device(p, ["grad"])
+            dev["grad"].add_(p.grad)
+        else:
+            dev["grad"] = p.grad
+            state["host_grad_valid"] = True
+        p.grad = None
+
+    def _maybe_warn_quant_master(self, state):
+        if self._quant_master_warned or state.get("master_filled") is not False:
+            return
+        warnings.warn("OffloadAdam: " + _LOSSY_MASTER_HINT, stacklevel=3)
+        self._quant_master_warned = True
+
+    def _call_step_fn(self, p, group, tensors, clip_coef=None):
+        state = self.state[p]
+        beta1, beta2 = group["betas"]
+        quant = p in self._quant_params
+        if quant:
+            self._maybe_warn_quant_master(state)
+        # A quantised weight cannot take the kernel's bf16 write-back: it goes to
+        # the gradient buffer (a sink) and the payload is re-encoded from the master.
+        self.step_fn(
+            tensors["grad"] if quant else p.data,
+            tensors,
+            group["lr"],
+            group["weight_decay"],
+            beta1,
+            beta2,
+            group["eps"],
+            state["step"],
+            decoupled_weight_decay=self.decoupled_weight_decay,
+            clip_coef=clip_coef,
+        )
+        if quant:
+            p.data.copy_(tensors["master_params"])
+
+    def _step_offload(self, p, group, clip_coef=None):
+        dev = self.device_states[p]
+        self._ensure_on_device(p, self.offload_state_keys)
+        self._call_step_fn(p, group, dev, clip_coef)
+        self._issue_d2h(p, self._non_grad_keys)
+        dev["grad"] = None
+
+    def _step_inplace(self, p, group, clip_coef=None):
+        state = self.state[p]
+        self._call_step_fn(p, group, {k: state[k] for k in self.offload_state_keys}, clip_coef)
+        state["grad"].zero_()
+
+    def _record_grad_norm(self, p, grad):
+        grad_clip.grad_norm_(grad.reshape(-1), self.state[p]["grad_norm"])
+
+    # ------------------------------------------------------------------ hooks
+
+    def _pre_backward_hook(self, module, grad_output):
+        # Idempotent across the several fires a backward can produce for one
+        # parameter (shared modules, tied weights): only what is not yet on the
+        # device is requested.
+        lazy = self._prefetch_policy == "lazy"
+        want_states = self._step_in_backward and self.ready_for_optimizer_step
+        for p in module.parameters():
+            if p in self._inplace_params or p not in self.device_states:
+                continue
+            if lazy and self._prefetch_module.get(p) is not module:
+                continue
+            dev = self.device_states[p]
+            keys = []
+            if self.state[p]["host_grad_valid"] and dev.get("grad") is None:
+                keys.append("grad")
+            if want_states:
+                keys += [k for k in self._non_grad_keys if dev.get(k) is None]
+            if keys:
+                self._issue_h2d(p, keys)
+
+    @torch.no_grad()
+    def _grad_hook(self, p):
+        if p.grad is None:
+            return
+        self._accumulate_grad_on_device(p)
+        state = self.state[p]
+        last = self.ready_for_optimizer_step
+        if self.max_grad_norm is not None and last:
+            self._record_grad_norm(p, self.device_states[p]["grad"])
+        if self._step_in_backward and last:
+            state["step"] += 1
+            self._step_offload(p, self._param2group[p])
+            state["host_grad_valid"] = False
+        else:
+            self._issue_d2h(p, ["grad"])
+
+    @torch.no_grad()
+    def _inplace_grad_hook(self, p):
+        if p.grad is None:
+            return
+        state = self.state[p]
+        state["grad"].add_(p.grad)
+        p.grad = None
+        last = self.ready_for_optimizer_step
+        if self.max_grad_norm is not None and last:
+            self._record_grad_norm(p, state["grad"])
+        if self._step_in_backward and last:
+            state["step"] += 1
+            self._step_inplace(p, self._param2group[p])
+
+    # ------------------------------------------------------------- public API
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        if closure is not None:
+            raise NotImplementedError(
+                "OffloadAdam does not support closure-based step: gradients are consumed by "
+                "backward hooks, so re-running backward inside a closure would corrupt "
+                "optimizer state."
+            )
+        if self._step_in_backward:
+            return
+
+        clip_coef = None
+        if self.max_grad_norm is not None:
+            grad_clip.clip_coef_(self._norm_slots, float(self.max_grad_norm), self._clip_coef,
+                                 self._total_norm)
+            clip_coef = self._clip_coef
+
+        order = [(g, p) for g in self.param_groups for p in g["params"]]
+        offloaded = [p for _, p in order if p not in self._inplace_params]
+        ahead = 0  # offloaded params whose H2D has been issued
+        done = 0
+        for group, p in order:
+            state = self.state[p]
+            state["step"] += 1
+            if p in self._inplace_params:
+                self._step_inplace(p, group, clip_coef)
+                continue
+            # keep the H2D engine a few parameters ahead of the kernels
+            while ahead < min(done + 1 + self._CLIP_PREFETCH_DEPTH, len(offloaded)):
+                q = offloaded[ahead]
+                dev = self.device_states[q]
+                missing = [k for k in self.offload_state_keys if dev.get(k) is None]
+                if missing:
+                    self._issue_h2d(q, missing)
+                ahead += 1
+            self._step_offload(p, group, clip_coef)
+            state["host_grad_valid"] = False
+            done += 1
+
+    def zero_grad(self, set_to_none=False):
+        """No-op: gradients are consumed by the hooks."""
+        return
+
+    @torch.no_grad()
+    def load_master_state_dict(self, state_dict, model, strict=False):
+        """Overwrite ``master_params`` from a ``{param_name: tensor}`` mapping (any
+        float dtype).  Returns ``(unexpected_keys,)``; ``strict=True`` raises
+        ``ValueError`` for names that match no parameter of this optimizer."""
+        if "master_params" not in self.offload_config:
+            raise RuntimeError(
+                "load_master_state_dict requires a mode that maintains master_params "
+                f"(e.g. 'fp32_master'); current mode is {self.mode!r}."
+            )
+        by_name = {n: p for n, p in model.named_parameters() if p.requires_grad}
+        unexpected = []
+        for name, tensor in state_dict.items():
+            p = by_name.get(name)
+            if p is None or p not in self.state:
+                unexpected.append(name)
+                continue
+            self._copy_master(p, tensor)
+            if "master_filled" in self.state[p]:
+                self.state[p]["master_filled"] = True
+        if strict and unexpected:
+            raise ValueError(
+                f"load_master_state_dict(strict=True): no param matches {len(unexpected)} "
+                f"key(s): {unexpected}"
+            )
+        return (unexpected,)
+
+    @torch.no_grad()
+    def load_master_from_pretrained(self, pretrained_name_or_path, model, *, strict=False):
+        """Refill the fp32 masters of quantised parameters from the bf16/fp16
+        checkpoint they were quantised from.  Returns the sorted names of
+        quantised parameters the checkpoint lacks."""
+        if "master_params" not in self.offload_config:
+            raise RuntimeError(
+                "load_master_from_pretrained requires a mode that maintains master_params "
+                f"(e.g. 'fp32_master'); current mode is {self.mode!r}."
+            )
+        return stream_master_from_pretrained(self, pretrained_name_or_path, model, strict=strict)
+
+    def load_state_dict(self, state_dict):
+        raise NotImplementedError(
+            "OffloadAdam.load_state_dict is not supported: the default "
+            "Optimizer.load_state_dict would move pinned-host state to GPU and cast fp32 "
+            "master to bf16, defeating the offload contract. File an issue if resume is needed."
+        )

@@ -1,0 +1,137 @@
+"""Exact-size pinned (page-locked) host tensors with an optional NUMA preference.
+
+Same surface as the reference's ``pinned_alloc`` module
+(src/offload_adam/pinned_alloc.py): ``zeros_pinned``, ``resolve_numa_target``,
+``numa_node_free_bytes``, ``gpu_numa_node``.  The memory comes from the HIP
+runtime through the library's ``oa_pinned_alloc`` (hipHostMalloc, rounded to
+4 KiB pages - no power-of-two rounding as in torch's pinned allocator), bound
+softly to a NUMA node with the thread memory policy, zero-filled by several
+threads, and released when the last tensor that views it is collected.
+"""
+
+import ctypes
+import os
+import weakref
+from pathlib import Path
+
+import torch
+
+from . import _lib
+
+_PAGE_SIZE = 4096
+_MPOL_SYSCALL_PROBED = None
+
+
+def _numa_policy_available():
+    """True when the kernel exposes NUMA nodes (memory policies can be applied)."""
+    global _MPOL_SYSCALL_PROBED
+    if _MPOL_SYSCALL_PROBED is None:
+        _MPOL_SYSCALL_PROBED = Path("/sys/devices/system/node/node0").exists()
+    return _MPOL_SYSCALL_PROBED
+
+
+def gpu_numa_node(device=None) -> int:
+    """NUMA node the given GPU hangs off, or -1 when the kernel reports none
+    (typical for single-socket hosts)."""
+    if device is None:
+        device = torch.cuda.current_device()
+    if isinstance(device, torch.device):
+        device = device.index if device.index is not None else torch.cuda.current_device()
+    node = ctypes.c_int(-1)
+    code = _lib.load().oa_gpu_numa_node(int(device), ctypes.byref(node))
+    if code != 0:
+        raise RuntimeError(f"HIP runtime error {code}: {_lib.error_string(code)}")
+    return node.value
+
+
+def resolve_numa_target(numa_node):
+    """Turn the user-facing ``numa_node`` knob into a node id or None.
+
+    * ``"auto"`` - the current GPU's node if the kernel knows it, else None.
+    * ``int``    - that node; raises when the host has no NUMA support.
+    * ``None``   - no binding.
+    """
+    if numa_node == "auto":
+        if torch.cuda.is_available() and _numa_policy_available():
+            detected = gpu_numa_node()
+            if detected >= 0:
+                return detected
+        return None
+    if isinstance(numa_node, int) and not isinstance(numa_node, bool):
+        if not _numa_policy_available():
+            raise RuntimeError(
+                "this host exposes no NUMA nodes; pass numa_node=None or 'auto'"
+            )
+        return numa_node
+    if numa_node is None:
+        return None
+    raise ValueError(f"numa_node must be 'auto', an int, or None (got {numa_node!r})")
+
+
+def numa_node_free_bytes(node: int):
+    """``MemFree`` of a NUMA node in bytes, or None if it cannot be read."""
+    try:
+        text = Path(f"/sys/devices/system/node/node{node}/meminfo").read_text()
+    except OSError:
+        return None
+    for line in text.splitlines():
+        if "MemFree:" in line:
+            return int(line.split()[-2]) * 1024  # "Node 1 MemFree:   64457228 kB"
+    return None
+
+
+def _alloc(size, numa_target):
+    """Page-locked, zero-filled allocation; returns (address, cleanup)."""
+    lib = _lib.load()
+    out = ctypes.c_void_p()
+    os_errno = ctypes.c_int(0)
+    code = lib.oa_pinned_alloc(
+        ctypes.c_size_t(size),
+        -1 if numa_target is None else int(numa_target),
+        ctypes.byref(out),
+        ctypes.byref(os_errno),
+    )
+    if code == _lib.OA_EOS:
+        err = os_errno.value
+        raise OSError(err, f"set_mempolicy(node={numa_target}) failed: {os.strerror(err)}")
+    if code != 0:
+        raise RuntimeError(
+            f"pinned allocation of {size} bytes failed with code {code}: "
+            f"{_lib.error_string(code)}"
+        )
+    ptr = out.value
+
+    def cleanup():
+        try:
+            lib.oa_pinned_free(ctypes.c_void_p(ptr))
+        except Exception:
+            pass
+
+    return ptr, cleanup
+
+
+def zeros_pinned(shape, dtype, numa_node="auto"):
+    """Zero-initialised pinned CPU tensor of exactly ``shape`` / ``dtype``.
+
+    ``numa_node``: ``"auto"`` (the GPU's node when known), an int node id, or
+    None.  The backing pages are freed when the last reference is dropped.
+    """
+    if torch.cuda.is_available():
+        torch.cuda.init()
+    shape = torch.Size(shape)
+    elem_size = torch.empty(0, dtype=dtype).element_size()
+    nbytes = shape.numel() * elem_size
+    size = ((nbytes + _PAGE_SIZE - 1) // _PAGE_SIZE) * _PAGE_SIZE
+    if size == 0:
+        size = _PAGE_SIZE
+
+    target = resolve_numa_target(numa_node)
+    ptr, cleanup = _alloc(size, target)
+    try:
+        buf = (ctypes.c_uint8 * size).from_address(ptr)
+        flat = torch.frombuffer(buf, dtype=torch.uint8)
+        weakref.finalize(flat.untyped_storage(), cleanup)
+        return flat.view(dtype)[: shape.numel()].view(shape)
+    except BaseException:
+        cleanup()
+        raise

@@ -1,0 +1,419 @@
+"""GPU tests of the host driver: pinned allocator, H2D/D2H streaming with event
+fencing, hook-driven and one-shot (clipping) steps, state layout, QAT.
+
+The reference has no test of this part; what pins it here is equivalence:
+``OffloadAdam`` (states on the host, step inside backward hooks, transfers on
+side streams) must leave parameters and states BIT-IDENTICAL to ``Adam`` (states
+on the GPU, plain ``step()``), which itself is checked against the oracle in
+test_adam_kernels_gpu.py.  Any missing fence or stale buffer breaks equality.
+"""
+
+import gc
+import random
+import warnings
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+BF16 = torch.bfloat16
+MODES = ["stochastic_rounding", "fp32_master", "fp31_master", "fp32_master_custom_rounding"]
+
+
+class TinyNet(nn.Module):
+    """A few Linear / norm layers; sizes straddle the in-place threshold used below."""
+
+    def __init__(self, d=96, h=160, tied=False):
+        super().__init__()
+        self.emb = nn.Embedding(50, d)
+        self.blocks = nn.ModuleList(
+            [nn.ModuleDict({"norm": nn.LayerNorm(d), "up": nn.Linear(d, h), "down": nn.Linear(h, d)})
+             for _ in range(3)]
+        )
+        self.head = nn.Linear(d, 50, bias=False)
+        if tied:
+            self.head.weight = self.emb.weight
+
+    def forward(self, ids):
+        x = self.emb(ids)
+        for b in self.blocks:
+            x = x + b["down"](F.gelu(b["up"](b["norm"](x))))
+        return self.head(x)
+
+
+def make_model(seed=0, tied=False):
+    torch.manual_seed(seed)
+    return TinyNet(tied=tied).to(device="cuda", dtype=BF16)
+
+
+def batches(n, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, 50, (4, 16), generator=g).cuda() for _ in range(n)]
+
+
+def loss_of(model, ids):
+    return F.cross_entropy(model(ids).float().reshape(-1, 50), ids.reshape(-1))
+
+
+@pytest.fixture
+def fixed_seed(monkeypatch):
+    """Both optimizers draw the stochastic-rounding seed from random.getrandbits;
+    a constant makes their random bits identical whatever the parameter order."""
+    monkeypatch.setattr(random, "getrandbits", lambda k: 0x1234_5678_9ABC_DEF0)
+
+
+def run_reference_adam(mode, steps, ga, seed=0, tied=False, **kw):
+    from offload_adam_amd import Adam
+
+    model = make_model(seed, tied)
+    opt = Adam(model.parameters(), mode=mode, lr=1e-2, weight_decay=0.01, **kw)
+    data = batches(steps * ga)
+    for s in range(steps):
+        for mb in range(ga):
+            loss_of(model, data[s * ga + mb]).backward()  # grads accumulate in bf16
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    return model, opt
+
+
+def run_offload_adam(mode, steps, ga, seed=0, tied=False, threshold=5000, **kw):
+    from offload_adam_amd import OffloadAdam
+
+    model = make_model(seed, tied)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode=mode, lr=1e-2, weight_decay=0.01,
+                          inplace_param_threshold=threshold, **kw)
+    data = batches(steps * ga)
+    for s in range(steps):
+        for mb in range(ga):
+            opt.ready_for_optimizer_step = mb == ga - 1
+            loss_of(model, data[s * ga + mb]).backward()
+        opt.step()
+        opt.zero_grad()
+    torch.cuda.synchronize()
+    return model, opt
+
+
+def assert_same_params(a, b):
+    for (n1, p1), (n2, p2) in zip(a.named_parameters(), b.named_parameters()):
+        assert n1 == n2
+        assert torch.equal(p1.view(torch.int16), p2.view(torch.int16)), n1
+
+
+# ------------------------------------------------------------- pinned memory
+
+
+def test_zeros_pinned_invariants():
+    from offload_adam_amd.pinned_alloc import (gpu_numa_node, numa_node_free_bytes,
+                                               resolve_numa_target, zeros_pinned)
+
+    for shape, dtype in [((3, 5), torch.float32), ((1000, 1000), BF16), ((0,), torch.int16),
+                         ((4097,), torch.int16)]:
+        t = zeros_pinned(shape, dtype, numa_node="auto")
+        assert t.shape == torch.Size(shape) and t.dtype == dtype and t.device.type == "cpu"
+        assert t.data_ptr() % 4096 == 0
+        assert t.is_pinned()
+        assert not t.any()
+        t.fill_(1)  # writable
+    node = gpu_numa_node()
+    assert isinstance(node, int) and node >= -1
+    assert resolve_numa_target(None) is None
+    assert resolve_numa_target("auto") in (None, node)
+    with pytest.raises(ValueError):
+        resolve_numa_target("nearest")
+    with pytest.raises(ValueError):
+        zeros_pinned((4,), BF16, numa_node=1.5)
+    free0 = numa_node_free_bytes(0)
+    if free0 is not None:  # the host exposes NUMA nodes: an explicit node works
+        assert free0 > 0
+        t = zeros_pinned((1 << 20,), torch.float32, numa_node=0)
+        assert not t.any() and t.is_pinned()
+    assert numa_node_free_bytes(10_000) is None
+
+
+def test_pinned_memory_is_released():
+    from offload_adam_amd import _lib, pinned_alloc
+
+    lib = _lib.load()
+    real = lib.oa_pinned_free
+    freed = []
+
+    def spy(ptr):
+        freed.append(ptr.value if hasattr(ptr, "value") else ptr)
+        return real(ptr)
+
+    lib.oa_pinned_free = spy
+    try:
+        t = pinned_alloc.zeros_pinned((1 << 20,), torch.float32, numa_node=None)
+        ptr = t.data_ptr()
+        view = t[10:20]
+        del t
+        gc.collect()
+        assert freed == []  # a surviving view keeps the pages alive
+        view.fill_(3.0)
+        assert view.sum().item() == 30.0
+        del view
+        gc.collect()
+        assert freed == [ptr]  # released exactly once, when the last view died
+    finally:
+        lib.oa_pinned_free = real
+
+
+def test_async_copy_round_trip_with_event_fencing():
+    """H2D on one side stream, kernel on the compute stream, D2H on another."""
+    from offload_adam_amd import _lib
+    from offload_adam_amd.offload_adam import _copy_async
+    from offload_adam_amd.pinned_alloc import zeros_pinned
+
+    n = 8_000_000
+    host_in = zeros_pinned((n,), torch.float32, numa_node=None)
+    host_out = zeros_pinned((n,), torch.float32, numa_node=None)
+    host_in.copy_(torch.arange(n, dtype=torch.float32))
+    h2d, d2h = torch.cuda.Stream(), torch.cuda.Stream()
+    compute = torch.cuda.current_stream()
+    for rep in range(3):
+        dev = torch.empty(n, dtype=torch.float32, device="cuda")
+        h2d.wait_stream(compute)
+        _copy_async(dev, host_in, _lib.OA_COPY_H2D, h2d)
+        ev = h2d.record_event()
+        compute.wait_event(ev)
+        dev.mul_(2.0)
+        d2h.wait_stream(compute)
+        _copy_async(host_out, dev, _lib.OA_COPY_D2H, d2h)
+        dev.record_stream(d2h)
+        d2h.synchronize()
+        assert torch.equal(host_out, host_in * 2.0), rep
+
+
+# ------------------------------------------------------- optimizer equivalence
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("ga", [1, 3])
+def test_hook_path_equals_adam(fixed_seed, mode, ga):
+    ref_model, ref_opt = run_reference_adam(mode, steps=4, ga=ga, decoupled_weight_decay=True)
+    model, opt = run_offload_adam(mode, steps=4, ga=ga, decoupled_weight_decay=True)
+    assert len(opt._offload_params) > 0 and len(opt._inplace_params) > 0
+    assert_same_params(ref_model, model)
+    # states agree too (host-resident vs GPU-resident)
+    for (pr, p) in zip(ref_model.parameters(), model.parameters()):
+        for key in ref_opt.config["states"]:
+            a, b = ref_opt.state[pr][key].cpu(), opt.state[p][key].cpu()
+            if a.dtype == BF16:
+                a, b = a.view(torch.int16), b.view(torch.int16)
+            assert torch.equal(a, b), key
+        assert opt.state[p]["step"] == 4
+
+
+@pytest.mark.parametrize("policy", ["eager", "lazy"])
+def test_tied_weights_and_prefetch_policies(fixed_seed, policy):
+    ref_model, _ = run_reference_adam("fp32_master", steps=3, ga=2, tied=True)
+    model, opt = run_offload_adam("fp32_master", steps=3, ga=2, tied=True, prefetch_policy=policy)
+    assert_same_params(ref_model, model)
+    assert sum(1 for _ in opt.param_groups[0]["params"]) == len(list(model.parameters()))
+
+
+def test_everything_offloaded_and_everything_inplace(fixed_seed):
+    ref_model, _ = run_reference_adam("stochastic_rounding", steps=3, ga=2)
+    m0, o0 = run_offload_adam("stochastic_rounding", steps=3, ga=2, threshold=0)
+    m1, o1 = run_offload_adam("stochastic_rounding", steps=3, ga=2, threshold=10**9)
+    assert not o0._inplace_params and not o1._offload_params
+    assert_same_params(ref_model, m0)
+    assert_same_params(ref_model, m1)
+
+
+@pytest.mark.parametrize("mode", ["fp31_master", "stochastic_rounding", "fp32_master"])
+@pytest.mark.parametrize("ga", [1, 2])
+def test_clip_path_equals_manual_clip_then_adam(fixed_seed, mode, ga):
+    """max_grad_norm path == per-parameter bf16 norms -> global bf16 coefficient
+    -> grad.mul_(coef) (torch) -> Adam.step(), the sequence the reference runs."""
+    from offload_adam_amd import Adam
+    from offload_adam_amd.grad_clip import clip_coef_, grad_norm_
+
+    max_norm = 0.05  # small enough to clip on every step
+    steps = 3
+    model, opt = run_offload_adam(mode, steps=steps, ga=ga, max_grad_norm=max_norm)
+    assert float(opt._clip_coef) < 1.0
+
+    ref = make_model(0)
+    ref_opt = Adam(ref.parameters(), mode=mode, lr=1e-2, weight_decay=0.01)
+    params = list(ref.parameters())
+    norms = torch.zeros(len(params), dtype=BF16, device="cuda")
+    coef = torch.ones((), dtype=BF16, device="cuda")
+    data = batches(steps * ga)
+    for s in range(steps):
+        for mb in range(ga):
+            loss_of(ref, data[s * ga + mb]).backward()
+        for i, p in enumerate(params):
+            grad_norm_(p.grad.reshape(-1), norms[i])
+        clip_coef_(norms, max_norm, coef)
+        for p in params:
+            p.grad.mul_(coef)
+        ref_opt.step()
+        ref_opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    assert_same_params(ref, model)
+    assert torch.equal(norms.view(torch.int16), opt._norm_slots.view(torch.int16))
+
+
+def test_clip_not_triggered_is_identity(fixed_seed):
+    ref_model, _ = run_reference_adam("fp31_master", steps=2, ga=1)
+    model, opt = run_offload_adam("fp31_master", steps=2, ga=1, max_grad_norm=1e6)
+    assert float(opt._clip_coef) == 1.0
+    assert_same_params(ref_model, model)
+
+
+# ------------------------------------------------------------ layout, errors
+
+
+def test_state_layout_and_api_surface():
+    from offload_adam_amd import OffloadAdam
+
+    model = make_model()
+    opt = OffloadAdam(model, mode="fp32_master", max_grad_norm=1.0, inplace_param_threshold=5000,
+                      verbose=0)
+    assert opt.mode == "fp32_master" and opt.ready_for_optimizer_step is False
+    assert opt.offload_state_keys == ["grad", "exp_avg", "exp_avg_sq", "master_params"]
+    group = opt.param_groups[0]
+    assert {"lr", "betas", "eps", "weight_decay", "params"} <= set(group)
+    for p in group["params"]:
+        st = opt.state[p]
+        assert st["step"] == 0
+        assert st["grad_norm"].dim() == 0 and st["grad_norm"].is_cuda
+        if p in opt._inplace_params:
+            assert "host_grad_valid" not in st
+            assert all(st[k].is_cuda for k in opt.offload_state_keys)
+        else:
+            assert st["host_grad_valid"] is False
+            for k, dt in opt.offload_config.items():
+                assert st[k].device.type == "cpu" and st[k].is_pinned()
+                assert st[k].dtype == dt and st[k].shape == p.shape
+            assert torch.equal(st["master_params"], p.detach().float().cpu())
+    sd = opt.state_dict()
+    assert set(sd) == {"state", "param_groups"} and len(sd["state"]) == len(group["params"])
+    with pytest.raises(NotImplementedError):
+        opt.load_state_dict(sd)
+    with pytest.raises(NotImplementedError):
+        opt.step(closure=lambda: None)
+    assert opt.zero_grad() is None
+    with pytest.raises(ValueError):
+        OffloadAdam(make_model(), prefetch_policy="sometimes")
+    with pytest.raises(AssertionError):
+        OffloadAdam(make_model(), mode="fp64_master")
+    with pytest.raises(RuntimeError):
+        OffloadAdam(make_model(), mode="stochastic_rounding").load_master_state_dict({}, model)
+
+
+def test_step_is_noop_in_hook_mode_and_returns_none():
+    from offload_adam_amd import OffloadAdam
+
+    model = make_model()
+    opt = OffloadAdam(model, inplace_param_threshold=5000)
+    before = [p.detach().clone() for p in model.parameters()]
+    assert opt.step() is None
+    for a, p in zip(before, model.parameters()):
+        assert torch.equal(a, p)
+
+
+# ----------------------------------------------------------------------- QAT
+
+
+@pytest.mark.parametrize("fmt", ["int8", "int4", "nf4", "nvfp4"])
+def test_qat_offload_equals_adam(fmt):
+    from offload_adam_amd import Adam, OffloadAdam
+    from offload_adam_amd.qweight import (Int4QWeight, Int8QWeight, NF4QWeight, NVFP4QWeight,
+                                          QWeightBase, quantize_linears)
+
+    cls, kw = {"int8": (Int8QWeight, {}), "int4": (Int4QWeight, {"group_size": 32}),
+               "nf4": (NF4QWeight, {"blocksize": 32}), "nvfp4": (NVFP4QWeight, {})}[fmt]
+
+    def build():
+        m = make_model()
+        report = quantize_linears(m, cls, skip_patterns=("head",), **kw)
+        assert len(report.quantized) == 6 and report.excluded == ["head"]
+        return m
+
+    data = batches(6)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        ref = build()
+        ref_opt = Adam(ref.parameters(), mode="fp32_master", lr=1e-2)
+        model = build()
+        opt = OffloadAdam(model, mode="fp32_master", lr=1e-2, inplace_param_threshold=5000)
+        assert len(opt._quant_params) == 6
+        for s in range(3):
+            for mb in range(2):
+                loss_of(ref, data[2 * s + mb]).backward()
+                opt.ready_for_optimizer_step = mb == 1
+                loss_of(model, data[2 * s + mb]).backward()
+            ref_opt.step()
+            ref_opt.zero_grad(set_to_none=True)
+            opt.step()
+    torch.cuda.synchronize()
+    for (n, pr), (_, p) in zip(ref.named_parameters(), model.named_parameters()):
+        if isinstance(p.data, QWeightBase):
+            for name in type(p.data)._PAYLOAD:
+                a, b = getattr(pr.data, name), getattr(p.data, name)
+                assert torch.equal(a.reshape(-1).view(torch.uint8),
+                                   b.reshape(-1).view(torch.uint8)), (n, name)
+            assert torch.equal(ref_opt.state[pr]["master_params"].cpu(),
+                               opt.state[p]["master_params"])
+            assert opt.state[p]["master_filled"] is False
+        else:
+            assert torch.equal(pr.view(torch.int16), p.view(torch.int16)), n
+    with pytest.raises(ValueError):
+        OffloadAdam(build(), mode="stochastic_rounding")
+
+
+def test_quant_master_warning_and_master_loading(tmp_path):
+    from safetensors.torch import save_file
+
+    from offload_adam_amd import OffloadAdam
+    from offload_adam_amd.qweight import Int8QWeight, quantize_linears
+
+    plain = make_model()
+    originals = {n: p.detach().clone() for n, p in plain.named_parameters()}
+    quantize_linears(plain, Int8QWeight, skip_patterns=("head",))
+    opt = OffloadAdam(plain, mode="fp32_master", inplace_param_threshold=5000)
+    q_names = [n for n, p in plain.named_parameters() if p in opt._quant_params]
+    # lossy seed: master == dequantised weight, flagged
+    p0 = dict(plain.named_parameters())[q_names[0]]
+    assert opt.state[p0]["master_filled"] is False
+    assert torch.equal(opt.state[p0]["master_params"], p0.data.dequantize().float().cpu())
+    opt.ready_for_optimizer_step = True
+    with pytest.warns(UserWarning, match="lossy dequant-seeded"):
+        loss_of(plain, batches(1)[0]).backward()
+    # lossless refill from a checkpoint of the original bf16 weights
+    ckpt = tmp_path / "model.safetensors"
+    save_file({n: t.cpu().contiguous() for n, t in originals.items()}, str(ckpt))
+    missing = opt.load_master_from_pretrained(str(ckpt), plain, strict=True)
+    assert missing == []
+    for n in q_names[1:]:
+        p = dict(plain.named_parameters())[n]
+        assert opt.state[p]["master_filled"] is True
+    unexpected, = opt.load_master_state_dict({"nope": torch.zeros(1)}, plain)
+    assert unexpected == ["nope"]
+    with pytest.raises(ValueError):
+        opt.load_master_state_dict({"nope": torch.zeros(1)}, plain, strict=True)
+
+
+def test_adam_state_dict_round_trip_keeps_fp32_master():
+    from offload_adam_amd import Adam
+
+    model = make_model()
+    opt = Adam(model.parameters(), mode="fp32_master", lr=1e-2)
+    loss_of(model, batches(1)[0]).backward()
+    opt.step()
+    sd = opt.state_dict()
+    opt2 = Adam(make_model().parameters(), mode="fp32_master", lr=1e-2)
+    opt2.load_state_dict(sd)
+    for p, p2 in zip(opt.param_groups[0]["params"], opt2.param_groups[0]["params"]):
+        assert opt2.state[p2]["master_params"].dtype == torch.float32
+        assert torch.equal(opt.state[p]["master_params"], opt2.state[p2]["master_params"])
+        assert opt2.state[p2]["step"] == 1
