@@ -155,6 +155,11 @@ def main():
     ap.add_argument("--workload", default="c1_sr_llama1b", choices=sorted(WORKLOADS))
     ap.add_argument("--rng", default=None, choices=[None, "triton", "x8"],
                     help="stochastic_rounding bit layout (default: the optimizer's own, x8)")
+    ap.add_argument("--per-tensor", action="store_true",
+                    help="one launch per tensor (the hook-path call pattern) instead of the "
+                         "multi-tensor launch")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run three 1 GiB device copies first (reference for counter runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-events", action="store_true",
                     help="skip per-launch HIP events (used for profiler runs)")
@@ -168,6 +173,8 @@ def main():
     import torch
 
     from offload_adam_amd import _lib, kernels
+    from offload_adam_amd.kernels import adam_step_multi
+    from offload_adam_amd.kernels.multi import MULTI_MAX
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -183,12 +190,29 @@ def main():
     clip = torch.tensor(0.3359375, dtype=torch.bfloat16, device=dev) if wl["clip"] else None
     total_elems = sum(p.numel() for p, _ in tensors)
     bytes_per_step = total_elems * BYTES_PER_ELEM[mode]
-    kw = {}
+    kw, multi_kw = {}, {}
     if mode == "stochastic_rounding" and args.rng is not None:
         kw["rng"] = args.rng
         kw["seed"] = 1
+        multi_kw["rng"] = args.rng
+        multi_kw["seeds"] = list(range(1, len(tensors) + 1))
+
+    multi = not args.per_tensor
+    p_list = [p for p, _ in tensors]
+    st_list = [st for _, st in tensors]
+    launches_per_step = -(-len(tensors) // MULTI_MAX) if multi else len(tensors)
 
     def one_step(step_no, events=None):
+        """One pass of the fused AdamW kernel over every tensor of the workload."""
+        if multi:
+            if events is not None:
+                events[0][0].record()
+            adam_step_multi(mode, p_list, st_list, 1e-4, 0.01, 0.9, 0.999, 1e-8, step_no,
+                            decoupled_weight_decay=True, clip_coef=clip, validate=False,
+                            **multi_kw)
+            if events is not None:
+                events[0][1].record()
+            return
         for i, (p, st) in enumerate(tensors):
             if events is not None:
                 events[i][0].record()
@@ -197,27 +221,38 @@ def main():
             if events is not None:
                 events[i][1].record()
 
+    if args.copy_calibration:
+        # A plain device copy of known size (1 GiB read + 1 GiB written), so a
+        # counter run can scale FETCH_SIZE / WRITE_SIZE to bytes.
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     for w in range(args.warmup):
         one_step(w + 1)
     torch.cuda.synchronize()
 
     # Timed region: exactly --steps steps, bracketed by device synchronisation.
+    # Events are recorded on the stream the kernels run on (torch's current
+    # stream) and read back after the closing synchronisation.
     use_events = not args.no_events
-    ev = None
-    kernel_ms = 0.0
-    launches = 0
+    pairs_per_step = 1 if multi else len(tensors)
+    all_events = []
     t0 = time.perf_counter()
     for s in range(args.steps):
+        ev = None
         if use_events:
             ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-                  for _ in tensors]
+                  for _ in range(pairs_per_step)]
+            all_events.append(ev)
         one_step(args.warmup + s + 1, ev)
-        if use_events:
-            torch.cuda.synchronize()
-            kernel_ms += sum(a.elapsed_time(b) for a, b in ev)
-            launches += len(ev)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    kernel_ms = sum(a.elapsed_time(b) for ev in all_events for a, b in ev)
+    launches = launches_per_step * len(all_events)
 
     ms_per_step = elapsed / args.steps * 1e3
     value = bytes_per_step * args.steps / elapsed / 1e9
@@ -225,11 +260,11 @@ def main():
     roofline = None
     if use_events and launches:
         avg_launch_s = kernel_ms / launches / 1e3
-        alg_bytes_per_launch = bytes_per_step / len(tensors)
+        alg_bytes_per_launch = bytes_per_step / launches_per_step
         achieved = alg_bytes_per_launch / avg_launch_s / 1e9
         roofline = {
             "bound": "hbm",
-            "kernel": f"adam_vec_kernel<{mode}>",
+            "kernel": f"{'adam_multi_kernel' if multi else 'adam_vec_kernel'}<{mode}>",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -260,6 +295,7 @@ def main():
             "elements": total_elems,
             "alg_bytes_per_elem": BYTES_PER_ELEM[mode],
             "resident": "HBM",
+            "launch": "multi_tensor" if multi else "per_tensor",
             "rng": kw.get("rng", "x8") if mode == "stochastic_rounding" else None,
         },
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),

@@ -134,6 +134,35 @@ int oa_adam_fp32_master_custom_rounding(void* param, const void* grad,
                                         float eps, int decoupled,
                                         const void* clip_coef, void* stream);
 
+/* Multi-tensor form of the four step functions: what a loop over parameters
+ * such as Adam.step (src/offload_adam/adam.py:111-152) or the in-place branch
+ * of OffloadAdam.step (src/offload_adam/offload_adam.py:563-571) does with one
+ * step_fn call per parameter, done with one launch per 36 parameters (tensor
+ * descriptors travel as kernel arguments; nothing is allocated).
+ *   mode        OA_MODE_*
+ *   count       number of parameters; every array below has `count` entries
+ *   params, grads, exp_avgs, exp_avg_sqs   device pointers, as in the
+ *               single-tensor entry points (for OA_MODE_FP32_MASTER params[i] is
+ *               the write-only bf16 sink and may equal grads[i])
+ *   aux         f32 masters (FP32_MASTER) or i16 rounding errors (FP31, CUSTOM);
+ *               ignored (may be NULL) for STOCHASTIC_ROUNDING
+ *   numels      element counts
+ *   beta1_hats, beta2_hats   per parameter (their step counts may differ)
+ *   seeds       per parameter, STOCHASTIC_ROUNDING only (else may be NULL)
+ *   rng         OA_RNG_TRITON or OA_RNG_X8 (STOCHASTIC_ROUNDING only)
+ * Every argument is validated before the first launch.  Results are identical
+ * to `count` single-tensor calls. */
+#define OA_MODE_FP32_MASTER         0
+#define OA_MODE_STOCHASTIC_ROUNDING 1
+#define OA_MODE_FP31_MASTER         2
+#define OA_MODE_CUSTOM_ROUNDING     3
+int oa_adam_multi(int mode, int count, void* const* params, const void* const* grads,
+                  void* const* exp_avgs, void* const* exp_avg_sqs, void* const* aux,
+                  const int64_t* numels, const float* beta1_hats,
+                  const float* beta2_hats, const uint64_t* seeds, float lr,
+                  float weight_decay, float eps, int decoupled, int rng,
+                  const void* clip_coef, void* stream);
+
 /* ------------------------------------------------------------------------
  * B. Gradient L2 norm per parameter and the global clip coefficient.
  * ---------------------------------------------------------------------- */

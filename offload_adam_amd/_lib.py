@@ -37,6 +37,13 @@ SIGNATURES = {
         c_int,
         [c_void_p] * 5 + _ADAM_TAIL + [c_void_p, c_void_p],
     ),
+    # mode, count, 5 pointer tables, numels, beta1_hats, beta2_hats, seeds,
+    # lr, wd, eps, decoupled, rng, clip_coef, stream
+    "oa_adam_multi": (
+        c_int,
+        [c_int, c_int] + [c_void_p] * 9 + [c_float, c_float, c_float, c_int, c_int, c_void_p,
+                                           c_void_p],
+    ),
     "oa_norm_workspace_bytes": (c_size_t, []),
     "oa_grad_norm_bf16": (
         c_int,

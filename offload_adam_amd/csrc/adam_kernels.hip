@@ -177,13 +177,12 @@ adam_scalar_kernel(const AdamArgs a) {
 // 16-bit arrays travel as four packed dwords (element 2j in the low half of
 // dword j), which is also the layout the hardware bf16 convert produces.
 template <int MODE, bool DEC, bool CLIP, int RNG>
-__global__ void __launch_bounds__(OA_ADAM_THREADS)
-adam_vec_kernel(const AdamArgs a) {
+__device__ __forceinline__ void adam_tile(const AdamArgs& a, int64_t tile, bool last_tile) {
   constexpr int T = OA_ADAM_THREADS;
   constexpr int U = OA_ADAM_UNROLL;
   const int64_t n_groups = a.n >> 3;
   const float clip = CLIP ? bf16_bits_to_f32(*a.clip) : 1.0f;
-  const int64_t g0 = (int64_t)blockIdx.x * (T * U) + threadIdx.x;
+  const int64_t g0 = tile * (T * U) + threadIdx.x;
 
   u32x4 P[U], G[U], Mo[U], Vo[U], R[U], E[U];
   f32x4 Ma[U], Mb[U];
@@ -287,11 +286,66 @@ adam_vec_kernel(const AdamArgs a) {
       st(reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.aux) + e0), En);
   }
 
-  // Tail: the last n % 8 elements, one lane each, in the last block.
-  if (blockIdx.x == gridDim.x - 1) {
+  // Tail: the last n % 8 elements, one lane each, in the tensor's last tile.
+  if (last_tile) {
     const int64_t i = (n_groups << 3) + threadIdx.x;
     if (i < a.n) adam_scalar<MODE, DEC, CLIP, RNG>(i, clip, a);
   }
+}
+
+template <int MODE, bool DEC, bool CLIP, int RNG>
+__global__ void __launch_bounds__(OA_ADAM_THREADS)
+adam_vec_kernel(const AdamArgs a) {
+  adam_tile<MODE, DEC, CLIP, RNG>(a, blockIdx.x, blockIdx.x == gridDim.x - 1);
+}
+
+// Multi-tensor form: one launch covers up to kMultiMax parameters.  The
+// per-tensor pointers and scalars travel in the kernel arguments (no device
+// table, nothing to allocate); block b finds its tensor by scanning the
+// prefix sums of tiles, which is uniform per block.  Back-to-back tensors share
+// one grid, so the ramp-up and drain of a launch are paid once per chunk
+// instead of once per parameter.
+constexpr int kMultiMax = 36;
+
+struct MultiArgs {
+  uint16_t* p[kMultiMax];
+  const uint16_t* g[kMultiMax];
+  uint16_t* m[kMultiMax];
+  uint16_t* v[kMultiMax];
+  void* aux[kMultiMax];
+  int64_t n[kMultiMax];
+  uint32_t tile_start[kMultiMax + 1];
+  float omb1[kMultiMax], omb2[kMultiMax];
+  uint32_t k0[kMultiMax], k1[kMultiMax];
+  const uint16_t* clip;
+  float lr, wd, lr_wd, eps;
+  int count;
+};
+
+template <int MODE, bool DEC, bool CLIP, int RNG>
+__global__ void __launch_bounds__(OA_ADAM_THREADS)
+adam_multi_kernel(const MultiArgs ma) {
+  int t = 0;
+  while (t + 1 < ma.count && blockIdx.x >= ma.tile_start[t + 1]) ++t;
+  AdamArgs a;
+  a.p = ma.p[t];
+  a.g = ma.g[t];
+  a.m = ma.m[t];
+  a.v = ma.v[t];
+  a.aux = ma.aux[t];
+  a.rand16 = nullptr;
+  a.clip = ma.clip;
+  a.n = ma.n[t];
+  a.lr = ma.lr;
+  a.wd = ma.wd;
+  a.lr_wd = ma.lr_wd;
+  a.omb1 = ma.omb1[t];
+  a.omb2 = ma.omb2[t];
+  a.eps = ma.eps;
+  a.k0 = ma.k0[t];
+  a.k1 = ma.k1[t];
+  const uint32_t tile = blockIdx.x - ma.tile_start[t];
+  adam_tile<MODE, DEC, CLIP, RNG>(a, tile, blockIdx.x + 1 == ma.tile_start[t + 1]);
 }
 
 template <int MODE, bool DEC, bool CLIP, int RNG>
@@ -459,4 +513,144 @@ extern "C" int oa_adam_fp32_master_custom_rounding(
   const bool vec = all16(param, grad, exp_avg, exp_avg_sq, rounding_error, nullptr);
   return dispatch_flags<kCustom, OA_RNG_TRITON>(a, decoupled != 0, vec,
                                                 static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------------------------ multi-tensor
+
+namespace oa {
+namespace {
+
+template <int MODE, int RNG>
+int launch_multi(const MultiArgs& ma, bool dec, unsigned tiles, hipStream_t s) {
+  const bool clip = ma.clip != nullptr;
+#define OA_LAUNCH_MULTI(D, C)                                                            \
+  hipLaunchKernelGGL((adam_multi_kernel<MODE, D, C, RNG>), dim3(tiles),                   \
+                     dim3(OA_ADAM_THREADS), 0, s, ma)
+  if (dec) {
+    if (clip) OA_LAUNCH_MULTI(true, true); else OA_LAUNCH_MULTI(true, false);
+  } else {
+    if (clip) OA_LAUNCH_MULTI(false, true); else OA_LAUNCH_MULTI(false, false);
+  }
+#undef OA_LAUNCH_MULTI
+  return launch_status();
+}
+
+int launch_multi_mode(int mode, int rng, const MultiArgs& ma, bool dec, unsigned tiles,
+                      hipStream_t s) {
+  switch (mode) {
+    case OA_MODE_FP32_MASTER:
+      return launch_multi<kFp32Master, OA_RNG_TRITON>(ma, dec, tiles, s);
+    case OA_MODE_STOCHASTIC_ROUNDING:
+      return rng == OA_RNG_X8 ? launch_multi<kStochastic, OA_RNG_X8>(ma, dec, tiles, s)
+                              : launch_multi<kStochastic, OA_RNG_TRITON>(ma, dec, tiles, s);
+    case OA_MODE_FP31_MASTER:
+      return launch_multi<kFp31, OA_RNG_TRITON>(ma, dec, tiles, s);
+    default:
+      return launch_multi<kCustom, OA_RNG_TRITON>(ma, dec, tiles, s);
+  }
+}
+
+}  // namespace
+}  // namespace oa
+
+extern "C" int oa_adam_multi(int mode, int count, void* const* params,
+                             const void* const* grads, void* const* exp_avgs,
+                             void* const* exp_avg_sqs, void* const* aux,
+                             const int64_t* numels, const float* beta1_hats,
+                             const float* beta2_hats, const uint64_t* seeds, float lr,
+                             float weight_decay, float eps, int decoupled, int rng,
+                             const void* clip_coef, void* stream) {
+  if (mode < OA_MODE_FP32_MASTER || mode > OA_MODE_CUSTOM_ROUNDING || count < 0)
+    return OA_EINVAL;
+  if (count == 0) return 0;
+  if (!params || !grads || !exp_avgs || !exp_avg_sqs || !numels || !beta1_hats || !beta2_hats)
+    return OA_EINVAL;
+  const bool has_aux = mode != OA_MODE_STOCHASTIC_ROUNDING;
+  const bool is_sr = mode == OA_MODE_STOCHASTIC_ROUNDING;
+  if (has_aux && !aux) return OA_EINVAL;
+  if (is_sr && (!seeds || (rng != OA_RNG_TRITON && rng != OA_RNG_X8))) return OA_EINVAL;
+  const size_t aux_align = mode == OA_MODE_FP32_MASTER ? 4 : 2;
+  // Validate everything before the first launch.
+  for (int i = 0; i < count; ++i) {
+    int rc = check_common(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i],
+                          has_aux ? aux[i] : nullptr, has_aux, aux_align, numels[i],
+                          clip_coef, mode == OA_MODE_FP32_MASTER);
+    if (rc) return rc;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool dec = decoupled != 0;
+  constexpr int64_t kPerTile = (int64_t)OA_ADAM_THREADS * OA_ADAM_UNROLL * 8;
+
+  MultiArgs ma;
+  ma.clip = static_cast<const uint16_t*>(clip_coef);
+  ma.lr = lr;
+  ma.wd = weight_decay;
+  volatile float lr_wd = lr * weight_decay;
+  ma.lr_wd = lr_wd;
+  ma.eps = eps;
+  ma.count = 0;
+  ma.tile_start[0] = 0;
+  uint64_t tiles = 0;
+
+  auto flush = [&]() -> int {
+    if (ma.count == 0) return 0;
+    int rc = launch_multi_mode(mode, rng, ma, dec, (unsigned)tiles, s);
+    ma.count = 0;
+    tiles = 0;
+    return rc;
+  };
+
+  for (int i = 0; i < count; ++i) {
+    const int64_t n = numels[i];
+    if (n == 0) continue;
+    void* ax = has_aux ? aux[i] : nullptr;
+    if (!all16(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i], ax, nullptr)) {
+      // not 16-byte aligned: single-tensor scalar path, in order
+      int rc = flush();
+      if (rc) return rc;
+      AdamArgs a = make_args(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i], ax, n, lr,
+                             weight_decay, beta1_hats[i], beta2_hats[i], eps, clip_coef);
+      if (is_sr) {
+        a.k0 = (uint32_t)(seeds[i] & 0xFFFFFFFFull);
+        a.k1 = (uint32_t)(seeds[i] >> 32);
+      }
+      switch (mode) {
+        case OA_MODE_FP32_MASTER:
+          rc = dispatch_flags<kFp32Master, OA_RNG_TRITON>(a, dec, false, s); break;
+        case OA_MODE_STOCHASTIC_ROUNDING:
+          rc = rng == OA_RNG_X8 ? dispatch_flags<kStochastic, OA_RNG_X8>(a, dec, false, s)
+                                : dispatch_flags<kStochastic, OA_RNG_TRITON>(a, dec, false, s);
+          break;
+        case OA_MODE_FP31_MASTER:
+          rc = dispatch_flags<kFp31, OA_RNG_TRITON>(a, dec, false, s); break;
+        default:
+          rc = dispatch_flags<kCustom, OA_RNG_TRITON>(a, dec, false, s); break;
+      }
+      if (rc) return rc;
+      continue;
+    }
+    int64_t t_tiles = (n + kPerTile - 1) / kPerTile;
+    if (t_tiles > 0x7FFFFFFFll) return OA_ERANGE;
+    if (ma.count == kMultiMax || tiles + (uint64_t)t_tiles > 0x7FFFFFFFull) {
+      int rc = flush();
+      if (rc) return rc;
+    }
+    const int j = ma.count;
+    ma.p[j] = static_cast<uint16_t*>(params[i]);
+    ma.g[j] = static_cast<const uint16_t*>(grads[i]);
+    ma.m[j] = static_cast<uint16_t*>(exp_avgs[i]);
+    ma.v[j] = static_cast<uint16_t*>(exp_avg_sqs[i]);
+    ma.aux[j] = ax;
+    ma.n[j] = n;
+    volatile float o1 = 1.0f - beta1_hats[i];
+    volatile float o2 = 1.0f - beta2_hats[i];
+    ma.omb1[j] = o1;
+    ma.omb2[j] = o2;
+    ma.k0[j] = is_sr ? (uint32_t)(seeds[i] & 0xFFFFFFFFull) : 0u;
+    ma.k1[j] = is_sr ? (uint32_t)(seeds[i] >> 32) : 0u;
+    tiles += (uint64_t)t_tiles;
+    ma.tile_start[j + 1] = (uint32_t)tiles;
+    ma.count = j + 1;
+  }
+  return flush();
 }

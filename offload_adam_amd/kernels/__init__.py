@@ -3,6 +3,7 @@
 from .fp31_master import adam_step_fp31_master
 from .fp32_master import adam_step_fp32_master
 from .fp32_master_custom_rounding import adam_step_fp32_master_custom_rounding
+from .multi import adam_step_multi
 from .stochastic_rounding import adam_step_stochastic_rounding
 
 __all__ = [
@@ -10,4 +11,5 @@ __all__ = [
     "adam_step_fp31_master",
     "adam_step_fp32_master",
     "adam_step_stochastic_rounding",
+    "adam_step_multi",
 ]

@@ -30,6 +30,7 @@ from torch.optim.optimizer import Optimizer
 from . import _lib, grad_clip
 from ._pretrained import stream_master_from_pretrained
 from .adam import _LOSSY_MASTER_HINT, MODE_TABLE
+from .kernels import adam_step_multi
 from .pinned_alloc import numa_node_free_bytes, resolve_numa_target, zeros_pinned
 from .qweight.base import QWeightBase
 
@@ -370,6 +371,30 @@ class OffloadAdam(Optimizer):
         self._call_step_fn(p, group, {k: state[k] for k in self.offload_state_keys}, clip_coef)
         state["grad"].zero_()
 
+    def _step_inplace_batch(self, params, group, clip_coef=None):
+        """``_step_inplace`` for a list of parameters with one multi-tensor launch."""
+        beta1, beta2 = group["betas"]
+        tensors, steps = [], []
+        for p in params:
+            state = self.state[p]
+            state["step"] += 1
+            steps.append(state["step"])
+            tensors.append({k: state[k] for k in self.offload_state_keys})
+        adam_step_multi(
+            self.mode,
+            [p.data for p in params],
+            tensors,
+            group["lr"],
+            group["weight_decay"],
+            beta1,
+            beta2,
+            group["eps"],
+            steps,
+            decoupled_weight_decay=self.decoupled_weight_decay,
+            clip_coef=clip_coef,
+        )
+        torch._foreach_zero_([t["grad"] for t in tensors])
+
     def _record_grad_norm(self, p, grad):
         grad_clip.grad_norm_(grad.reshape(-1), self.state[p]["grad_norm"])
 
@@ -448,12 +473,16 @@ class OffloadAdam(Optimizer):
         offloaded = [p for _, p in order if p not in self._inplace_params]
         ahead = 0  # offloaded params whose H2D has been issued
         done = 0
+        # GPU-resident small parameters: one multi-tensor launch per group
+        for group in self.param_groups:
+            small = [p for p in group["params"] if p in self._inplace_params]
+            if small:
+                self._step_inplace_batch(small, group, clip_coef)
         for group, p in order:
+            if p in self._inplace_params:
+                continue
             state = self.state[p]
             state["step"] += 1
-            if p in self._inplace_params:
-                self._step_inplace(p, group, clip_coef)
-                continue
             # keep the H2D engine a few parameters ahead of the kernels
             while ahead < min(done + 1 + self._CLIP_PREFETCH_DEPTH, len(offloaded)):
                 q = offloaded[ahead]

@@ -256,6 +256,59 @@ def test_multi_step_trajectory(oracle):
                 sc["rounding_error"] = torch.from_numpy(ref["rounding_error"].copy())
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("clip", [None, 0.3359375])
+def test_multi_tensor_equals_single_calls(oracle, mode, clip):
+    """One multi-tensor call over 80 tensors (three launch chunks, sizes from 1
+    element to 300k, one unaligned view, per-tensor step counts and seeds) leaves
+    every tensor exactly as the oracle's per-tensor result."""
+    from offload_adam_amd.kernels import adam_step_multi
+
+    rng = np.random.default_rng(0)
+    sizes = [1, 7, 8, 2048, 2049, 300_001] + [int(s) for s in rng.integers(1, 50_000, 74)]
+    params, states, steps, seeds, refs = [], [], [], [], []
+    clip_t = None if clip is None else torch.tensor(clip, dtype=torch.bfloat16, device="cuda")
+    clip_bits = None if clip is None else int(bits(clip_t.reshape(1))[0])
+    for i, n in enumerate(sizes):
+        off = 1 if i == 5 else 0  # one tensor off the 16-byte boundary
+        p0, st0 = adam_inputs(n + off, seed=100 + i, mode=mode, device="cuda")
+        p, st = p0[off:], {k: v[off:] for k, v in st0.items()}
+        step, seed = 1 + i % 7, 1000 + i
+        refs.append(_oracle_step(oracle, mode, p, st, True, clip_bits, seed=seed, layout=0,
+                                 hyp=dict(HYP, step=step)))
+        params.append(p)
+        states.append(st)
+        steps.append(step)
+        seeds.append(seed)
+    kw = dict(seeds=seeds, rng="triton") if mode == "stochastic_rounding" else {}
+    adam_step_multi(mode, params, states, HYP["lr"], HYP["weight_decay"], HYP["beta1"],
+                    HYP["beta2"], HYP["eps"], steps, decoupled_weight_decay=True,
+                    clip_coef=clip_t, **kw)
+    torch.cuda.synchronize()
+    for i, (p, st, ref) in enumerate(zip(params, states, refs)):
+        _assert_equal(mode, p, st, ref, f"multi {mode} tensor {i} n={sizes[i]}")
+
+
+def test_multi_tensor_rejects_before_launching():
+    from offload_adam_amd import _lib
+    from offload_adam_amd.kernels import adam_step_multi
+
+    p, st = adam_inputs(64, seed=1, mode="fp31_master", device="cuda")
+    before = bits(p)
+    bad = dict(st, exp_avg=st["exp_avg"][:8])
+    with pytest.raises(ValueError):
+        adam_step_multi("fp31_master", [p, p], [st, bad], 1e-3, 0.0, 0.9, 0.999, 1e-8, 1)
+    with pytest.raises(ValueError):
+        adam_step_multi("fp99", [p], [st], 1e-3, 0.0, 0.9, 0.999, 1e-8, 1)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(p), before)
+    lib = _lib.load()
+    assert lib.oa_adam_multi(9, 1, None, None, None, None, None, None, None, None, None,
+                             0, 0, 0, 0, 0, None, None) == -1
+    assert lib.oa_adam_multi(0, 0, None, None, None, None, None, None, None, None, None,
+                             0, 0, 0, 0, 0, None, None) == 0
+
+
 def test_argument_errors():
     from offload_adam_amd import _lib
 
