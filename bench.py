@@ -24,6 +24,15 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE counter runs of this script, each scaled by what the same counter
+# read for a 1 GiB device copy (factors 2.000 and 1.000).  Keyed by
+# (workload, launch form); the summary with the commands is
+# profiles/adam_multi_kernel_sr_c1_llama1b_hbm_traffic.txt.
+MEASURED_TRAFFIC_BYTES = {
+    ("c1_sr_llama1b", "multi_tensor"): 2_566_900_000,
+}
+
 BYTES_PER_ELEM = {
     "stochastic_rounding": 14,
     "fp32_master": 20,
@@ -269,7 +278,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(
+                (args.workload, "multi_tensor" if multi else "per_tensor")),
             "alg_bytes_per_launch": int(alg_bytes_per_launch),
             "avg_launch_us": round(avg_launch_s * 1e6, 2),
             "launches": launches,
