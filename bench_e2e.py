@@ -1,0 +1,303 @@
+#!/usr/bin/env python3
+"""End-to-end synthetic training step with OffloadAdam on one MI355X
+(BASELINE config 4) and the host-link measurements that go with it.
+
+    python bench_e2e.py [--model llama8b|llama1b|tiny] [--steps K] [--warmup W]
+                        [--grad-accum 4] [--seq 4096] [--mode stochastic_rounding]
+
+Model: a Llama-style decoder written here in plain PyTorch (RMSNorm, rotary
+embeddings, grouped-query SDPA attention, SwiGLU MLP, untied embeddings), bf16,
+random init, per-layer activation checkpointing.  Data: uniform random token
+ids.  The loop has the shape of the reference's example
+(examples/e2e_train/train.py:183-213): for each micro-batch set
+``optimizer.ready_for_optimizer_step``, forward, backward; then
+``optimizer.step()``.
+
+Reported: step time, tokens/s, the same loop with no optimizer (pure
+forward/backward) to expose the optimizer's non-overlapped cost, bytes moved
+over the host link per step and the achieved H2D / D2H rates against the pinned
+``hipMemcpyAsync`` peak measured in the same run.  Prints ONE JSON line.
+"""
+
+import argparse
+import json
+import math
+import sys
+import time
+import warnings
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+MODELS = {
+    # BASELINE config 4 / config 2 shapes
+    "llama8b": dict(hidden=4096, inter=14336, layers=32, q_heads=32, kv_heads=8, head_dim=128,
+                    vocab=128256),
+    # BASELINE config 1 shapes
+    "llama1b": dict(hidden=2048, inter=5632, layers=22, q_heads=32, kv_heads=4, head_dim=64,
+                    vocab=32000),
+    "tiny": dict(hidden=256, inter=688, layers=2, q_heads=4, kv_heads=2, head_dim=64, vocab=1024),
+}
+
+
+def build_model(cfg, device):
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    from torch.utils.checkpoint import checkpoint
+
+    class RMSNorm(nn.Module):
+        def __init__(self, dim, eps=1e-5):
+            super().__init__()
+            self.weight = nn.Parameter(torch.ones(dim))
+            self.eps = eps
+
+        def forward(self, x):
+            v = x.float()
+            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + self.eps)
+            return (v * self.weight.float()).to(x.dtype)
+
+    def rotary(x, cos, sin):
+        x1, x2 = x[..., ::2], x[..., 1::2]
+        return torch.stack((x1 * cos - x2 * sin, x1 * sin + x2 * cos), dim=-1).flatten(-2)
+
+    class Block(nn.Module):
+        def __init__(self, c):
+            super().__init__()
+            h, hd = c["hidden"], c["head_dim"]
+            self.nq, self.nkv, self.hd = c["q_heads"], c["kv_heads"], hd
+            self.input_layernorm = RMSNorm(h)
+            self.q_proj = nn.Linear(h, self.nq * hd, bias=False)
+            self.k_proj = nn.Linear(h, self.nkv * hd, bias=False)
+            self.v_proj = nn.Linear(h, self.nkv * hd, bias=False)
+            self.o_proj = nn.Linear(self.nq * hd, h, bias=False)
+            self.post_attention_layernorm = RMSNorm(h)
+            self.gate_proj = nn.Linear(h, c["inter"], bias=False)
+            self.up_proj = nn.Linear(h, c["inter"], bias=False)
+            self.down_proj = nn.Linear(c["inter"], h, bias=False)
+
+        def forward(self, x, cos, sin):
+            b, s, _ = x.shape
+            y = self.input_layernorm(x)
+            q = self.q_proj(y).view(b, s, self.nq, self.hd).transpose(1, 2)
+            k = self.k_proj(y).view(b, s, self.nkv, self.hd).transpose(1, 2)
+            v = self.v_proj(y).view(b, s, self.nkv, self.hd).transpose(1, 2)
+            q, k = rotary(q, cos, sin), rotary(k, cos, sin)
+            rep = self.nq // self.nkv
+            if rep > 1:
+                k = k.repeat_interleave(rep, dim=1)
+                v = v.repeat_interleave(rep, dim=1)
+            a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+            x = x + self.o_proj(a.transpose(1, 2).reshape(b, s, self.nq * self.hd))
+            y = self.post_attention_layernorm(x)
+            return x + self.down_proj(F.silu(self.gate_proj(y)) * self.up_proj(y))
+
+    class Decoder(nn.Module):
+        def __init__(self, c):
+            super().__init__()
+            self.c = c
+            self.embed_tokens = nn.Embedding(c["vocab"], c["hidden"])
+            self.layers = nn.ModuleList([Block(c) for _ in range(c["layers"])])
+            self.norm = RMSNorm(c["hidden"])
+            self.lm_head = nn.Linear(c["hidden"], c["vocab"], bias=False)
+
+        def forward(self, ids):
+            s = ids.shape[1]
+            hd = self.c["head_dim"]
+            inv = 1.0 / (500000.0 ** (torch.arange(0, hd, 2, device=ids.device).float() / hd))
+            ang = torch.arange(s, device=ids.device).float()[:, None] * inv[None, :]
+            cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+            x = self.embed_tokens(ids)
+            for layer in self.layers:
+                x = checkpoint(layer, x, cos, sin, use_reentrant=False)
+            x = self.norm(x)
+            # cross-entropy in sequence chunks: the fp32 logits of 4096 x 128256 stay bounded
+            loss = x.new_zeros((), dtype=torch.float32)
+            chunk = 1024
+            tgt = torch.roll(ids, -1, dims=1)
+            for i in range(0, s, chunk):
+                logits = self.lm_head(x[:, i:i + chunk]).float()
+                loss = loss + F.cross_entropy(logits.reshape(-1, logits.shape[-1]),
+                                              tgt[:, i:i + chunk].reshape(-1), reduction="sum")
+            return loss / ids.numel()
+
+    with torch.device(device):
+        model = Decoder(cfg).to(torch.bfloat16)
+    g = torch.Generator(device=device).manual_seed(0)
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() > 1:
+                p.normal_(0.0, 0.02, generator=g)
+    return model
+
+
+def measure_link(nbytes=1 << 30, reps=5):
+    """Pinned hipMemcpyAsync rates of this box: H2D alone, D2H alone, both at once."""
+    import torch
+
+    from offload_adam_amd import _lib
+    from offload_adam_amd.offload_adam import _copy_async
+    from offload_adam_amd.pinned_alloc import zeros_pinned
+
+    host_a = zeros_pinned((nbytes,), torch.uint8)
+    host_b = zeros_pinned((nbytes,), torch.uint8)
+    dev_a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    dev_b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+
+    def run(h2d, d2h):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            if h2d:
+                _copy_async(dev_a, host_a, _lib.OA_COPY_H2D, s1)
+            if d2h:
+                _copy_async(host_b, dev_b, _lib.OA_COPY_D2H, s2)
+        s1.synchronize()
+        s2.synchronize()
+        return nbytes * reps / (time.perf_counter() - t0) / 1e9
+
+    def run_mixed(wg):
+        """H2D on the DMA engine while the copy kernel writes back (the pairing
+        the optimizer uses)."""
+        from offload_adam_amd.offload_adam import _copy_by_kernel
+
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            _copy_async(dev_a, host_a, _lib.OA_COPY_H2D, s1)
+            _copy_by_kernel(host_b, dev_b, s2, wg)
+        s1.synchronize()
+        s2.synchronize()
+        return nbytes * reps / (time.perf_counter() - t0) / 1e9
+
+    run(True, True)  # warm-up
+    return {
+        "h2d_GBps": round(run(True, False), 2),
+        "d2h_GBps": round(run(False, True), 2),
+        "bidir_each_GBps": round(run(True, True), 2),
+        "dma_h2d_plus_kernel_d2h_each_GBps": {wg: round(run_mixed(wg), 2) for wg in (4, 8, 16)},
+    }
+
+
+def link_bytes_per_step(opt, grad_accum):
+    """Bytes the hook path moves per optimizer step for the offloaded parameters."""
+    import torch
+
+    n = sum(p.numel() for p in opt._offload_params)
+    state_b = sum(torch.empty(0, dtype=d).element_size()
+                  for k, d in opt.offload_config.items() if k != "grad")
+    if opt._step_in_backward:
+        h2d = n * (2 * (grad_accum - 1) + state_b)
+        d2h = n * (2 * (grad_accum - 1) + state_b)
+    else:
+        h2d = n * (2 * (grad_accum - 1) + 2 + state_b)
+        d2h = n * (2 * grad_accum + state_b)
+    return h2d, d2h
+
+
+def run(args):
+    import torch
+
+    from offload_adam_amd import OffloadAdam, _lib
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = MODELS[args.model]
+    out = {"model": args.model, "mode": args.mode, "seq": args.seq, "batch": 1,
+           "grad_accum": args.grad_accum, "max_grad_norm": args.max_grad_norm}
+
+    out["link_peak"] = measure_link()
+
+    model = build_model(cfg, dev)
+    n_params = sum(p.numel() for p in model.parameters())
+    out["params"] = n_params
+    ids = [torch.randint(0, cfg["vocab"], (1, args.seq), device=dev,
+                         generator=torch.Generator(device=dev).manual_seed(i))
+           for i in range(args.grad_accum)]
+
+    def loop(opt, steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            for mb in range(args.grad_accum):
+                if opt is not None:
+                    opt.ready_for_optimizer_step = mb == args.grad_accum - 1
+                loss = model(ids[mb])
+                loss.backward()
+                if opt is None:
+                    model.zero_grad(set_to_none=True)
+            if opt is not None:
+                opt.step()
+                opt.zero_grad()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    # 1) forward/backward only: what a step costs with a free optimizer
+    loop(None, 1)
+    out["fwd_bwd_only_s"] = round(loop(None, args.steps), 4)
+
+    # 2) the offloaded optimizer
+    t0 = time.perf_counter()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, lr=1e-5, mode=args.mode, max_grad_norm=args.max_grad_norm,
+                          inplace_param_threshold=1024 * 1024, prefetch_policy="eager",
+                          decoupled_weight_decay=True)
+    torch.cuda.synchronize()
+    out["optimizer_init_s"] = round(time.perf_counter() - t0, 2)
+    out["offloaded_params"] = len(opt._offload_params)
+    out["inplace_params"] = len(opt._inplace_params)
+    out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
+
+    torch.cuda.reset_peak_memory_stats()
+    loop(opt, args.warmup)
+    step_s = loop(opt, args.steps)
+    out["step_s"] = round(step_s, 4)
+    out["tokens_per_s"] = round(args.grad_accum * args.seq / step_s, 1)
+    out["exposed_optimizer_s"] = round(step_s - out["fwd_bwd_only_s"], 4)
+    out["peak_gpu_GiB"] = round(torch.cuda.max_memory_allocated() / 1024**3, 2)
+    h2d, d2h = link_bytes_per_step(opt, args.grad_accum)
+    out["h2d_GB_per_step"] = round(h2d / 1e9, 2)
+    out["d2h_GB_per_step"] = round(d2h / 1e9, 2)
+    out["h2d_GBps_over_step"] = round(h2d / step_s / 1e9, 2)
+    out["d2h_GBps_over_step"] = round(d2h / step_s / 1e9, 2)
+    peak = out["link_peak"]["bidir_each_GBps"]
+    out["link_floor_s"] = round(max(h2d, d2h) / 1e9 / peak, 4)
+    out["loss_finite"] = bool(math.isfinite(float(model(ids[0]))))
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--model", default="llama8b", choices=sorted(MODELS))
+    ap.add_argument("--mode", default="stochastic_rounding")
+    ap.add_argument("--seq", type=int, default=4096)
+    ap.add_argument("--grad-accum", type=int, default=4)
+    ap.add_argument("--max-grad-norm", type=float, default=None)
+    ap.add_argument("--steps", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--d2h-workgroups", type=int, default=None,
+                    help="workgroups of the write-back copy kernel (default: the optimizer's)")
+    ap.add_argument("--one-transfer-stream", action="store_true")
+    ap.add_argument("--prefetch-gib", type=float, default=None,
+                    help="device staging budget of the H2D prefetch window")
+    args = ap.parse_args()
+    if args.one_transfer_stream or args.prefetch_gib:
+        from offload_adam_amd import offload_adam as _oa_mod
+
+        _oa_mod._ONE_TRANSFER_STREAM = args.one_transfer_stream
+        if args.prefetch_gib:
+            _oa_mod.OffloadAdam._PREFETCH_BYTES = int(args.prefetch_gib * 2**30)
+    if args.d2h_workgroups:
+        from offload_adam_amd import offload_adam as _oa_mod
+
+        _oa_mod._D2H_BY_KERNEL = True
+        _oa_mod._D2H_WORKGROUPS = args.d2h_workgroups
+    print(json.dumps(run(args)))
+
+
+if __name__ == "__main__":
+    main()

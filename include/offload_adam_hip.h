@@ -305,6 +305,18 @@ int oa_gpu_numa_node(int device, int* node_out);
 #define OA_COPY_D2D 2
 int oa_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream);
 
+/* The same copy done by a small grid-stride kernel (`workgroups` blocks of 1024
+ * lanes, 128-bit accesses, 4 loads in flight per lane; 8 blocks fill a PCIe
+ * Gen5 x16 link) instead of the DMA engine.  Either pointer may be
+ * page-locked host memory from oa_pinned_alloc: the lanes read or write it
+ * across the host link.  Used for one direction of the streaming path so that
+ * H2D (DMA engine) and D2H (this kernel) never queue behind each other on one
+ * engine.  Both pointers must be 16-byte aligned.  No counterpart in the
+ * reference (its copies all go through `Tensor.to` / `copy_`,
+ * src/offload_adam/offload_adam.py:347-372). */
+int oa_copy_kernel_async(void* dst, const void* src, size_t bytes, int workgroups,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

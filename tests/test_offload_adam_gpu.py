@@ -191,6 +191,45 @@ def test_async_copy_round_trip_with_event_fencing():
         assert torch.equal(host_out, host_in * 2.0), rep
 
 
+@pytest.mark.parametrize("nbytes", [16, 4096 + 7, 3 * (1 << 20) + 5, 64 << 20])
+@pytest.mark.parametrize("workgroups", [1, 8])
+def test_copy_kernel_moves_exact_bytes(nbytes, workgroups):
+    """oa_copy_kernel_async: host->device and device->host, byte tail included."""
+    from offload_adam_amd import _lib
+    from offload_adam_amd.pinned_alloc import zeros_pinned
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(nbytes)
+    host_in = zeros_pinned((nbytes + 16,), torch.uint8, numa_node=None)
+    host_out = zeros_pinned((nbytes + 16,), torch.uint8, numa_node=None)
+    host_in.copy_(torch.randint(0, 256, (nbytes + 16,), dtype=torch.uint8, generator=g))
+    dev = torch.full((nbytes + 16,), 0xAA, dtype=torch.uint8, device="cuda")
+    s = _lib.current_stream_ptr()
+    _lib.check(lib.oa_copy_kernel_async(_lib.ptr(dev), _lib.ptr(host_in), nbytes, workgroups, s),
+               "h2d")
+    _lib.check(lib.oa_copy_kernel_async(_lib.ptr(host_out), _lib.ptr(dev), nbytes, workgroups, s),
+               "d2h")
+    torch.cuda.synchronize()
+    assert torch.equal(dev[:nbytes].cpu(), host_in[:nbytes])
+    assert (dev[nbytes:] == 0xAA).all()  # nothing written past the byte count
+    assert torch.equal(host_out[:nbytes], host_in[:nbytes])
+    assert (host_out[nbytes:] == 0).all()
+    # argument checks
+    assert lib.oa_copy_kernel_async(_lib.ptr(dev), _lib.ptr(host_in), nbytes, 0, s) == -1
+    assert lib.oa_copy_kernel_async(dev.data_ptr() + 4, _lib.ptr(host_in), nbytes, 1, s) == -2
+    assert lib.oa_copy_kernel_async(None, None, 0, 1, s) == 0
+
+
+def test_d2h_by_kernel_switch_gives_identical_results(fixed_seed, monkeypatch):
+    """The write-back path by copy kernel is a transport choice only."""
+    from offload_adam_amd import offload_adam as oa_mod
+
+    ref_model, _ = run_offload_adam("stochastic_rounding", steps=3, ga=2)
+    monkeypatch.setattr(oa_mod, "_D2H_BY_KERNEL", True)
+    model, _ = run_offload_adam("stochastic_rounding", steps=3, ga=2)
+    assert_same_params(ref_model, model)
+
+
 # ------------------------------------------------------- optimizer equivalence
 
 
