@@ -200,7 +200,7 @@ def link_bytes_per_step(opt, grad_accum):
 def run(args):
     import torch
 
-    from offload_adam_amd import OffloadAdam, _lib
+    from offload_adam_amd import OffloadAdam, _copy_engines, _lib  # before any CUDA call
 
     _lib.load()
     dev = torch.device("cuda:0")
@@ -266,6 +266,9 @@ def run(args):
     out["d2h_GBps_over_step"] = round(d2h / step_s / 1e9, 2)
     peak = out["link_peak"]["bidir_each_GBps"]
     out["link_floor_s"] = round(max(h2d, d2h) / 1e9 / peak, 4)
+    st = _copy_engines.status()
+    out["copy_engines"] = {k: st.get(k) for k in ("loaded", "active", "h2d_engine", "d2h_engine",
+                                                  "h2d_copies", "d2h_copies", "rejected")}
     out["loss_finite"] = bool(math.isfinite(float(model(ids[0]))))
     return out
 
@@ -284,7 +287,14 @@ def main():
     ap.add_argument("--one-transfer-stream", action="store_true")
     ap.add_argument("--prefetch-gib", type=float, default=None,
                     help="device staging budget of the H2D prefetch window")
+    ap.add_argument("--runtime-copy-engines", action="store_true",
+                    help="leave the SDMA engine of each copy to the HIP runtime "
+                         "(do not load the fixed-engine tools library)")
     args = ap.parse_args()
+    if args.runtime_copy_engines:
+        import os
+
+        os.environ["OFFLOAD_ADAM_COPY_ENGINES"] = "off"  # before the package is imported
     if args.one_transfer_stream or args.prefetch_gib:
         from offload_adam_amd import offload_adam as _oa_mod
 

@@ -1,0 +1,46 @@
+/* liboffload_adam_copy_engines.so: an HSA tools library (loaded by the ROCr
+ * runtime through HSA_TOOLS_LIB, before the first HIP call) that gives the
+ * host->device and the device->host copies of the process one fixed SDMA
+ * engine each.  It has no counterpart in the reference, whose copies go
+ * through torch's non_blocking copies on two CUDA streams
+ * (src/offload_adam/offload_adam.py:346-358 and :362-372) and rely on the CUDA
+ * driver's copy engines; on MI355X the HIP runtime's per-copy engine choice has
+ * to be taken out of the picture to get a full-duplex host link.
+ *
+ * OnLoad / OnUnload are the entry points the ROCr runtime calls (tools
+ * interface of hsa_api_trace.h).  The functions below only report state; they
+ * may be called at any time, from any thread, by whoever dlopen()s the same
+ * file.
+ *
+ * Environment, read once when the runtime loads the library:
+ *   OFFLOAD_ADAM_COPY_ENGINES="<h2d mask>,<d2h mask>"  one bit each, values of
+ *       hsa_amd_sdma_engine_id_t; default "0x1,0x2" (SDMA engines 0 and 1)
+ *   OFFLOAD_ADAM_COPY_ENGINES=off                      rewrite nothing
+ */
+#ifndef OFFLOAD_ADAM_COPY_ENGINES_H
+#define OFFLOAD_ADAM_COPY_ENGINES_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* 1 once the ROCr runtime has called OnLoad in this process, else 0. */
+int oa_copy_engines_loaded(void);
+
+/* 1 while copies are being rewritten; 0 when switched off by configuration or
+ * after eight rewritten calls in a row were rejected by the runtime. */
+int oa_copy_engines_active(void);
+
+/* The engine masks in use (hsa_amd_sdma_engine_id_t values). */
+void oa_copy_engines_config(unsigned* h2d_mask, unsigned* d2h_mask);
+
+/* Copies issued on the fixed engines so far, per direction, and rewritten
+ * calls the runtime rejected (each of those was re-issued unchanged). */
+void oa_copy_engines_stats(unsigned long long* h2d_copies, unsigned long long* d2h_copies,
+                           unsigned long long* rejected);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* OFFLOAD_ADAM_COPY_ENGINES_H */

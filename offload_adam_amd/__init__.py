@@ -6,8 +6,14 @@ Public surface mirrors the reference package ``offload_adam``: ``Adam`` and
 ``offload_adam_amd.qweight``).
 """
 
-from .adam import Adam
-from .offload_adam import OffloadAdam
+from . import _copy_engines
+
+# Must run before the first HIP call of the process: it names the SDMA-engine
+# tools library in HSA_TOOLS_LIB, which the runtime reads while it initialises.
+_copy_engines.install()
+
+from .adam import Adam  # noqa: E402
+from .offload_adam import OffloadAdam  # noqa: E402
 
 __version__ = "0.1.0"
 

@@ -1,8 +1,12 @@
-"""Builds liboffload_adam_hip.so in-tree with hipcc for gfx950.
+"""Builds the package's two shared libraries in-tree.
 
-Run ``python -m offload_adam_amd._build`` (or call :func:`build_library`).
-The library is compiled once, ahead of time, on any machine with ROCm's
-hipcc (no GPU needed); nothing is compiled at import time.
+* ``liboffload_adam_hip.so`` - kernels and C ABI, hipcc for gfx950.
+* ``liboffload_adam_copy_engines.so`` - the HSA tools library that fixes the
+  SDMA engine of each copy direction; host-only C++.
+
+Run ``python -m offload_adam_amd._build`` (or call :func:`build_all`).  Both
+are compiled once, ahead of time, on any machine with ROCm (no GPU needed);
+nothing is compiled at import time.
 """
 
 import os
@@ -17,6 +21,8 @@ CSRC_DIR = PKG_DIR / "csrc"
 INCLUDE_DIR = PKG_DIR.parent / "include"
 LIB_NAME = "liboffload_adam_hip.so"
 LIB_PATH = PKG_DIR / LIB_NAME
+TOOL_SRC = CSRC_DIR / "hsa_tool" / "copy_engine_pin.cpp"
+TOOL_LIB_PATH = PKG_DIR / "liboffload_adam_copy_engines.so"
 OFFLOAD_ARCH = "gfx950"
 
 # -ffp-contract=off and correctly rounded divide/sqrt are part of the numeric
@@ -94,5 +100,35 @@ def build_library(extra_flags=(), verbose=True, jobs=None, out_path=None):
     return out_path
 
 
+def build_copy_engine_tool(verbose=True, out_path=None):
+    """Compile the HSA tools library.  It talks to the ROCr runtime only through
+    the API table it is handed at load, so it links against nothing."""
+    hipcc = _hipcc()
+    # a plain C++ compiler: the hipcc wrapper would link the HIP runtime in
+    cxx = shutil.which("g++") or shutil.which("amdclang++") or "/opt/rocm/bin/amdclang++"
+    rocm_include = Path(hipcc).resolve().parents[1] / "include"
+    if not (rocm_include / "hsa" / "hsa_api_trace.h").exists():
+        rocm_include = Path("/opt/rocm/include")
+    out_path = Path(out_path) if out_path else TOOL_LIB_PATH
+    tmp = out_path.with_suffix(".so.tmp")
+    # hsa_api_trace.h finds its sibling headers as "inc/..." unless
+    # AMD_INTERNAL_BUILD is defined; the installed tree has them side by side.
+    cmd = [cxx, "-O2", "-std=c++17", "-shared", "-fPIC", "-Wall",
+           "-DAMD_INTERNAL_BUILD", f"-I{rocm_include}", f"-I{rocm_include / 'hsa'}",
+           f"-I{INCLUDE_DIR}", str(TOOL_SRC), "-o", str(tmp)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"compiling {TOOL_SRC.name} failed:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, out_path)
+    return out_path
+
+
+def build_all(extra_flags=(), verbose=True, jobs=None):
+    return [build_library(extra_flags, verbose, jobs), build_copy_engine_tool(verbose)]
+
+
 if __name__ == "__main__":
-    print(build_library())
+    for path in build_all():
+        print(path)

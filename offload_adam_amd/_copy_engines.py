@@ -1,0 +1,74 @@
+"""Registration of liboffload_adam_copy_engines.so with the ROCr runtime.
+
+The library (csrc/hsa_tool/copy_engine_pin.cpp) gives host->device and
+device->host copies one fixed SDMA engine each.  The runtime loads tools
+libraries named in ``HSA_TOOLS_LIB`` while it initialises, which happens at the
+first HIP call of the process (for torch: the first CUDA call, not
+``import torch``).  :func:`install` therefore runs when the package is imported
+and only edits the environment; nothing is loaded here.
+
+``OFFLOAD_ADAM_COPY_ENGINES=off`` keeps the environment untouched.
+"""
+
+import ctypes
+import os
+import sys
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "liboffload_adam_copy_engines.so"
+
+_install_result = None
+
+
+def _gpu_runtime_started():
+    torch = sys.modules.get("torch")
+    try:
+        return bool(torch is not None and torch.cuda.is_initialized())
+    except Exception:
+        return False
+
+
+def install():
+    """Put the tools library on ``HSA_TOOLS_LIB``.  Returns one of
+    ``"installed"``, ``"off"`` (disabled by the environment), ``"missing"``
+    (library not built) or ``"late"`` (the GPU runtime is already up)."""
+    global _install_result
+    if _install_result in ("installed", "off"):
+        return _install_result
+    if os.environ.get("OFFLOAD_ADAM_COPY_ENGINES", "").strip().lower() in ("off", "0", "none"):
+        _install_result = "off"
+    elif not LIB_PATH.exists():
+        _install_result = "missing"
+    elif str(LIB_PATH) in os.environ.get("HSA_TOOLS_LIB", "").split():
+        _install_result = "installed"
+    elif _gpu_runtime_started():
+        _install_result = "late"
+    else:
+        current = os.environ.get("HSA_TOOLS_LIB", "").strip()
+        os.environ["HSA_TOOLS_LIB"] = (str(LIB_PATH) + " " + current).strip()
+        _install_result = "installed"
+    return _install_result
+
+
+def status():
+    """What the tools library reports once the GPU runtime is up:
+    ``{"install", "loaded", "active", "h2d_engine", "d2h_engine", "h2d_copies",
+    "d2h_copies", "rejected"}``.  ``loaded`` is False when the runtime started
+    before :func:`install` ran (or the library is missing)."""
+    out = {"install": _install_result, "loaded": False, "active": False}
+    if not LIB_PATH.exists():
+        return out
+    lib = ctypes.CDLL(str(LIB_PATH))  # same handle the runtime holds, if it loaded it
+    lib.oa_copy_engines_loaded.restype = ctypes.c_int
+    lib.oa_copy_engines_active.restype = ctypes.c_int
+    lib.oa_copy_engines_config.restype = None
+    lib.oa_copy_engines_stats.restype = None
+    out["loaded"] = bool(lib.oa_copy_engines_loaded())
+    out["active"] = bool(lib.oa_copy_engines_active())
+    h2d, d2h = ctypes.c_uint(0), ctypes.c_uint(0)
+    lib.oa_copy_engines_config(ctypes.byref(h2d), ctypes.byref(d2h))
+    out["h2d_engine"], out["d2h_engine"] = h2d.value, d2h.value
+    a, b, c = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
+    lib.oa_copy_engines_stats(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))
+    out["h2d_copies"], out["d2h_copies"], out["rejected"] = a.value, b.value, c.value
+    return out

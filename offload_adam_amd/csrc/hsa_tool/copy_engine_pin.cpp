@@ -1,0 +1,139 @@
+// HSA tools library: one fixed SDMA engine per direction of host<->device copies.
+//
+// Why it exists.  The HIP runtime issues pinned host<->device copies with
+// hsa_amd_memory_async_copy_on_engine and re-picks the engine of a stream from
+// hsa_amd_memory_copy_engine_status: the lowest engine that is idle at that
+// instant.  An engine counts as busy while this very stream's previous copy is
+// still running, so a stream that keeps its direction saturated walks up
+// through the engines.  On MI355X only SDMA engines 0-3 reach the host link's
+// rate (57 GB/s for a 117 MB copy: 2.1 ms); engines 4-7 take 9.2 ms for the same
+// copy, 8-11 take 11.7 ms and engine 12 takes 16.5 ms.  When the pick lands on
+// the engine the other direction uses, the two directions share one in-order
+// ring and the link runs half duplex.  A training step that streams optimizer
+// states both ways falls into both traps for hundreds of milliseconds at a time.
+//
+// What it does.  The ROCr runtime loads every library named in HSA_TOOLS_LIB
+// during hsa_init and hands it the API table.  OnLoad swaps the table's
+// hsa_amd_memory_async_copy_on_engine for a wrapper that rewrites the engine of
+// CPU->GPU copies to one fixed engine and of GPU->CPU copies to another.
+// Dependency and completion signals pass through untouched, so the HIP runtime's
+// stream ordering is unchanged; copies of one direction simply queue on one ring
+// in issue order.  GPU<->GPU copies and everything else are left alone.  If the
+// runtime rejects a rewritten call, the original call is made instead, and after
+// eight such rejections in a row the rewrite switches itself off.
+//
+// Configuration (read once, at load):
+//   OFFLOAD_ADAM_COPY_ENGINES="<h2d mask>,<d2h mask>"   default "0x1,0x2"
+//   OFFLOAD_ADAM_COPY_ENGINES=off                       load, but rewrite nothing
+//
+// The include directory of hsa_api_trace.h is laid out for ROCr's own build
+// unless AMD_INTERNAL_BUILD is defined; the build line defines it and adds
+// <rocm>/include/hsa to the include path.
+
+#include <hsa.h>
+#include <hsa_ext_amd.h>
+#include <hsa_api_trace.h>
+
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+
+#include "offload_adam_copy_engines.h"
+
+namespace {
+
+decltype(hsa_amd_memory_async_copy_on_engine)* real_copy_on_engine = nullptr;
+decltype(hsa_agent_get_info)* real_agent_get_info = nullptr;
+
+std::atomic<int> loaded{0};
+std::atomic<int> active{0};
+unsigned h2d_engine = 0x1;
+unsigned d2h_engine = 0x2;
+std::atomic<unsigned long long> n_h2d{0}, n_d2h{0}, n_rejected{0};
+std::atomic<int> rejected_in_a_row{0};
+constexpr int kMaxRejectedInARow = 8;
+
+bool single_bit(unsigned m) { return m != 0 && (m & (m - 1)) == 0 && m <= 0x8000u; }
+
+bool is_cpu(hsa_agent_t agent) {
+  hsa_device_type_t type = HSA_DEVICE_TYPE_GPU;
+  if (real_agent_get_info(agent, HSA_AGENT_INFO_DEVICE, &type) != HSA_STATUS_SUCCESS) return false;
+  return type == HSA_DEVICE_TYPE_CPU;
+}
+
+hsa_status_t copy_on_fixed_engine(void* dst, hsa_agent_t dst_agent, const void* src,
+                                  hsa_agent_t src_agent, size_t size, uint32_t num_dep_signals,
+                                  const hsa_signal_t* dep_signals, hsa_signal_t completion_signal,
+                                  hsa_amd_sdma_engine_id_t engine_id, bool force_copy_on_sdma) {
+  if (active.load(std::memory_order_relaxed)) {
+    const bool src_cpu = is_cpu(src_agent), dst_cpu = is_cpu(dst_agent);
+    unsigned want = 0;
+    if (src_cpu && !dst_cpu) want = h2d_engine;
+    else if (!src_cpu && dst_cpu) want = d2h_engine;
+    if (want != 0) {
+      hsa_status_t st = real_copy_on_engine(dst, dst_agent, src, src_agent, size, num_dep_signals,
+                                            dep_signals, completion_signal,
+                                            static_cast<hsa_amd_sdma_engine_id_t>(want),
+                                            force_copy_on_sdma);
+      if (st == HSA_STATUS_SUCCESS) {
+        (src_cpu ? n_h2d : n_d2h).fetch_add(1, std::memory_order_relaxed);
+        rejected_in_a_row.store(0, std::memory_order_relaxed);
+        return st;
+      }
+      n_rejected.fetch_add(1, std::memory_order_relaxed);
+      if (rejected_in_a_row.fetch_add(1, std::memory_order_relaxed) + 1 >= kMaxRejectedInARow)
+        active.store(0, std::memory_order_relaxed);
+    }
+  }
+  return real_copy_on_engine(dst, dst_agent, src, src_agent, size, num_dep_signals, dep_signals,
+                             completion_signal, engine_id, force_copy_on_sdma);
+}
+
+// "0x1,0x2" -> masks; anything malformed keeps the defaults.  Returns false for "off".
+bool read_config() {
+  const char* s = getenv("OFFLOAD_ADAM_COPY_ENGINES");
+  if (!s || !*s) return true;
+  if (!strcmp(s, "off") || !strcmp(s, "0") || !strcmp(s, "none")) return false;
+  char* end = nullptr;
+  unsigned long a = strtoul(s, &end, 0);
+  if (!end || *end != ',') return true;
+  unsigned long b = strtoul(end + 1, &end, 0);
+  if (single_bit((unsigned)a) && single_bit((unsigned)b)) {
+    h2d_engine = (unsigned)a;
+    d2h_engine = (unsigned)b;
+  }
+  return true;
+}
+
+}  // namespace
+
+extern "C" bool OnLoad(HsaApiTable* table, uint64_t /*runtime_version*/,
+                       uint64_t /*failed_tool_count*/, const char* const* /*failed_tool_names*/) {
+  if (!table || !table->core_ || !table->amd_ext_) return true;
+  if (!table->amd_ext_->hsa_amd_memory_async_copy_on_engine_fn) return true;
+  const bool rewrite = read_config();
+  real_agent_get_info = table->core_->hsa_agent_get_info_fn;
+  real_copy_on_engine = table->amd_ext_->hsa_amd_memory_async_copy_on_engine_fn;
+  table->amd_ext_->hsa_amd_memory_async_copy_on_engine_fn = copy_on_fixed_engine;
+  active.store(rewrite ? 1 : 0);
+  loaded.store(1);
+  return true;
+}
+
+extern "C" void OnUnload() { active.store(0); }
+
+extern "C" int oa_copy_engines_loaded(void) { return loaded.load(); }
+
+extern "C" int oa_copy_engines_active(void) { return active.load(); }
+
+extern "C" void oa_copy_engines_config(unsigned* h2d_mask, unsigned* d2h_mask) {
+  if (h2d_mask) *h2d_mask = h2d_engine;
+  if (d2h_mask) *d2h_mask = d2h_engine;
+}
+
+extern "C" void oa_copy_engines_stats(unsigned long long* h2d_copies, unsigned long long* d2h_copies,
+                                      unsigned long long* rejected) {
+  if (h2d_copies) *h2d_copies = n_h2d.load();
+  if (d2h_copies) *d2h_copies = n_d2h.load();
+  if (rejected) *rejected = n_rejected.load();
+}

@@ -27,7 +27,7 @@ from ctypes import c_int, c_size_t, c_void_p
 import torch
 from torch.optim.optimizer import Optimizer
 
-from . import _lib, grad_clip
+from . import _copy_engines, _lib, grad_clip
 from ._pretrained import stream_master_from_pretrained
 from .adam import _LOSSY_MASTER_HINT, MODE_TABLE
 from .kernels import adam_step_multi
@@ -62,6 +62,7 @@ def _copy_async(dst, src, kind, stream):
 
 
 _ONE_TRANSFER_STREAM = False  # queue both directions on one side stream
+_copy_engine_warned = False
 _D2H_BY_KERNEL = False  # write-back engine: DMA (default) or the library's copy kernel
 _D2H_WORKGROUPS = 8  # 1024-lane workgroups: enough requests in flight to fill the host link
 
@@ -190,6 +191,8 @@ class OffloadAdam(Optimizer):
         self.d2h_events = {}
         self.h2d_stream = torch.cuda.Stream()
         self.d2h_stream = self.h2d_stream if _ONE_TRANSFER_STREAM else torch.cuda.Stream()
+        if self._offload_params:
+            self._check_copy_engines()
         self._param2group = {p: g for g in self.param_groups for p in g["params"]}
         # first module in forward order that owns each offloaded param ('lazy' policy)
         self._prefetch_module = {}
@@ -307,6 +310,27 @@ class OffloadAdam(Optimizer):
     #   the compute stream waits for H2D(p) before touching p's device states;
     #   D2H(p) starts after everything the compute stream has enqueued so far;
     #   a device buffer is not recycled before the D2H that reads it is done.
+
+    def _check_copy_engines(self):
+        """Warn once when the fixed-engine tools library is not in effect: the HIP
+        runtime then picks an SDMA engine per copy, and the streaming step runs
+        half duplex with stretches of 10 GB/s write-back."""
+        global _copy_engine_warned
+        st = _copy_engines.status()
+        if st["loaded"] or st["install"] == "off" or _copy_engine_warned:
+            return
+        _copy_engine_warned = True
+        why = {
+            "late": "offload_adam_amd was imported after the GPU runtime had started",
+            "missing": f"{_copy_engines.LIB_PATH.name} is not built "
+                       "(python -m offload_adam_amd._build)",
+        }.get(st["install"], "the ROCr runtime did not load it from HSA_TOOLS_LIB")
+        warnings.warn(
+            "OffloadAdam: host<->device copies are not pinned to fixed SDMA engines ("
+            + why + "); expect a slower streaming step.  Import offload_adam_amd before "
+            "the first CUDA call, or set OFFLOAD_ADAM_COPY_ENGINES=off to silence this.",
+            stacklevel=3,
+        )
 
     def _host_view(self, p, name):
         return self.state[p][name]

@@ -17,6 +17,10 @@ def _has_gpu():
     try:
         import torch
 
+        # the package names its SDMA-engine tools library in HSA_TOOLS_LIB at
+        # import; that has to happen before the first call into the GPU runtime
+        import offload_adam_amd  # noqa: F401
+
         return torch.cuda.is_available()
     except Exception:
         return False

@@ -1,0 +1,105 @@
+"""The HSA tools library that fixes the SDMA engine per copy direction
+(include/offload_adam_copy_engines.h, csrc/hsa_tool/copy_engine_pin.cpp)."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "offload_adam_copy_engines.h"
+
+
+def declared():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(oa_copy_engines_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_header_symbols_and_tool_entry_points():
+    from offload_adam_amd import _copy_engines
+
+    assert _copy_engines.LIB_PATH.exists(), "build with `python -m offload_adam_amd._build`"
+    lib = ctypes.CDLL(str(_copy_engines.LIB_PATH))
+    names = declared()
+    assert names == ["oa_copy_engines_active", "oa_copy_engines_config", "oa_copy_engines_loaded",
+                     "oa_copy_engines_stats"]
+    for name in names + ["OnLoad", "OnUnload"]:
+        assert hasattr(lib, name), name
+
+
+def test_status_without_runtime_reports_not_loaded():
+    from offload_adam_amd import _copy_engines
+
+    st = _copy_engines.status()
+    if st["loaded"]:
+        pytest.skip("a GPU runtime is up in this process")
+    assert st["active"] is False
+    assert (st["h2d_engine"], st["d2h_engine"]) == (1, 2)
+    assert st["h2d_copies"] == st["d2h_copies"] == st["rejected"] == 0
+
+
+def _run(code, **env):
+    full = dict(os.environ)
+    full.pop("HSA_TOOLS_LIB", None)
+    full.pop("OFFLOAD_ADAM_COPY_ENGINES", None)
+    full.update(env)
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=full,
+                         cwd=str(ROOT), timeout=300)
+    assert res.returncode == 0, res.stderr
+    return res.stdout.strip().splitlines()[-1]
+
+
+def test_import_puts_library_on_hsa_tools_lib():
+    code = ("import os, offload_adam_amd; from offload_adam_amd import _copy_engines as c; "
+            "print(c._install_result, os.environ.get('HSA_TOOLS_LIB'))")
+    result, value = _run(code).split(" ", 1)
+    assert result == "installed" and value.endswith("liboffload_adam_copy_engines.so")
+    # an existing entry is kept, ours goes first
+    result, value = _run(code, HSA_TOOLS_LIB="/some/other/tool.so").split(" ", 1)
+    assert result == "installed"
+    assert value.split()[0].endswith("liboffload_adam_copy_engines.so")
+    assert value.split()[1] == "/some/other/tool.so"
+
+
+def test_off_leaves_environment_alone():
+    code = ("import os, offload_adam_amd; from offload_adam_amd import _copy_engines as c; "
+            "print(c._install_result, os.environ.get('HSA_TOOLS_LIB'))")
+    assert _run(code, OFFLOAD_ADAM_COPY_ENGINES="off") == "off None"
+
+
+@pytest.mark.gpu
+def test_copies_run_on_the_fixed_engines_and_move_the_right_bytes():
+    import torch
+
+    from offload_adam_amd import _copy_engines, _lib
+    from offload_adam_amd.offload_adam import _copy_async
+    from offload_adam_amd.pinned_alloc import zeros_pinned
+
+    torch.cuda.init()
+    st0 = _copy_engines.status()
+    assert st0["loaded"] and st0["active"], st0
+    n = 4 << 20
+    host_in = zeros_pinned((n,), torch.int32, numa_node=None)
+    host_out = zeros_pinned((n,), torch.int32, numa_node=None)
+    host_in.copy_(torch.arange(n, dtype=torch.int32))
+    h2d, d2h = torch.cuda.Stream(), torch.cuda.Stream()
+    main = torch.cuda.current_stream()
+    for rep in range(4):
+        dev = torch.empty(n, dtype=torch.int32, device="cuda")
+        h2d.wait_stream(main)
+        _copy_async(dev, host_in, _lib.OA_COPY_H2D, h2d)
+        main.wait_stream(h2d)
+        dev.add_(rep)
+        d2h.wait_stream(main)
+        _copy_async(host_out, dev, _lib.OA_COPY_D2H, d2h)
+        dev.record_stream(d2h)
+        d2h.synchronize()
+        assert torch.equal(host_out, host_in + rep)
+    st1 = _copy_engines.status()
+    assert st1["h2d_copies"] - st0["h2d_copies"] >= 4
+    assert st1["d2h_copies"] - st0["d2h_copies"] >= 4
+    assert st1["rejected"] == 0 and st1["active"]
