@@ -266,6 +266,7 @@ def run(args):
     out["d2h_GBps_over_step"] = round(d2h / step_s / 1e9, 2)
     peak = out["link_peak"]["bidir_each_GBps"]
     out["link_floor_s"] = round(max(h2d, d2h) / 1e9 / peak, 4)
+    out["transfer_streams"] = opt.transfer_stream_report
     st = _copy_engines.status()
     out["copy_engines"] = {k: st.get(k) for k in ("loaded", "active", "h2d_engine", "d2h_engine",
                                                   "h2d_copies", "d2h_copies", "rejected")}

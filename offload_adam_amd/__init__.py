@@ -6,11 +6,12 @@ Public surface mirrors the reference package ``offload_adam``: ``Adam`` and
 ``offload_adam_amd.qweight``).
 """
 
-from . import _copy_engines
+from . import _runtime_env
 
-# Must run before the first HIP call of the process: it names the SDMA-engine
-# tools library in HSA_TOOLS_LIB, which the runtime reads while it initialises.
-_copy_engines.install()
+# Must run before the first HIP call of the process: names the SDMA-engine tools
+# library in HSA_TOOLS_LIB and reserves hardware queues for the transfer streams;
+# the runtime reads both while it initialises.
+_runtime_env.prepare()
 
 from .adam import Adam  # noqa: E402
 from .offload_adam import OffloadAdam  # noqa: E402

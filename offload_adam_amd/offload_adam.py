@@ -21,6 +21,7 @@ What runs underneath is this package's HIP library: the fused AdamW kernels
 ``hipMemcpyAsync`` on two side streams fenced with events.
 """
 
+import time
 import warnings
 from ctypes import c_int, c_size_t, c_void_p
 
@@ -65,6 +66,109 @@ _ONE_TRANSFER_STREAM = False  # queue both directions on one side stream
 _copy_engine_warned = False
 _D2H_BY_KERNEL = False  # write-back engine: DMA (default) or the library's copy kernel
 _D2H_WORKGROUPS = 8  # 1024-lane workgroups: enough requests in flight to fill the host link
+
+
+_PROBE_TRANSFER_STREAMS = True
+_PROBE_MAX_CANDIDATES = 8
+_PROBE_PASS_RATIO = 0.85
+
+
+def _probe_concurrency(device, h2d, d2h, bufs, rounds=6):
+    """Time the optimizer's copy pattern on a candidate pair of side streams.
+
+    Returns ``(duplex, h2d_with_compute, d2h_with_compute)``: elapsed time of two
+    activities together divided by the sum of their times alone.  Measured
+    values: 0.59 (both directions) and 0.72 (a direction and kernels) when they
+    run side by side, 0.99-1.0 when one waits for the other.  Each copy is followed by
+    an event record and preceded by a fence on the compute stream, as in the
+    streaming step: those are what serialise streams that share a hardware
+    queue."""
+    host_in, host_out, dev_in, dev_out, x = bufs
+    compute = torch.cuda.current_stream(device)
+
+    def up():
+        h2d.wait_stream(compute)
+        _copy_async(dev_in, host_in, _lib.OA_COPY_H2D, h2d)
+        h2d.record_event()
+
+    def down():
+        d2h.wait_stream(compute)
+        _copy_async(host_out, dev_out, _lib.OA_COPY_D2H, d2h)
+        d2h.record_event()
+
+    def kernels():
+        for _ in range(6):
+            x.mul_(1.0)
+
+    def timed(*activities):
+        torch.cuda.synchronize(device)
+        t0 = time.perf_counter()
+        for _ in range(rounds):
+            for act in activities:
+                act()
+        torch.cuda.synchronize(device)
+        return time.perf_counter() - t0
+
+    timed(up, down, kernels)  # warm
+    t_up, t_down, t_k = timed(up), timed(down), timed(kernels)
+    duplex = timed(up, down) / (t_up + t_down)
+    # copy first: its fence covers the previous round's kernels, this round's run beside it
+    up_with_compute = timed(up, kernels) / (t_k + t_up)
+    down_with_compute = timed(down, kernels) / (t_k + t_down)
+    return duplex, up_with_compute, down_with_compute
+
+
+def pick_transfer_streams(device):
+    """Two side streams on which host->device copies, device->host copies and the
+    compute stream's kernels run concurrently.
+
+    HIP streams share a small pool of hardware queues (``GPU_MAX_HW_QUEUES``, 4
+    unless set before the HIP library loads); a new stream goes to the queue with
+    the fewest users.  When the two transfer streams land on one queue, or one of
+    them on the compute stream's, the event markers of one sit in the same
+    in-order queue as the fences of the other and the link runs half duplex
+    (measured on the 8B step: 3.1 s instead of 2.1 s).  Which queue a stream got
+    cannot be asked, so it is measured: candidates are drawn from torch's stream
+    pool until a pair passes, at most ``_PROBE_MAX_CANDIDATES`` streams.
+
+    Returns ``(h2d_stream, d2h_stream, report)``."""
+    nbytes = 32 << 20
+    bufs = (
+        zeros_pinned((nbytes,), torch.uint8, numa_node=None),
+        zeros_pinned((nbytes,), torch.uint8, numa_node=None),
+        torch.empty(nbytes, dtype=torch.uint8, device=device),
+        torch.zeros(nbytes, dtype=torch.uint8, device=device),
+        torch.zeros(128 << 20, dtype=torch.bfloat16, device=device),  # 0.1 ms per pass
+    )
+    with torch.cuda.device(device):
+        h2d, d2h = torch.cuda.Stream(device), torch.cuda.Stream(device)
+        tried, best = 2, None
+        while True:
+            duplex, up_c, down_c = _probe_concurrency(device, h2d, d2h, bufs)
+            with_compute = max(up_c, down_c)
+            score = max(duplex, with_compute)
+            if best is None or score < best[0]:
+                best = (score, h2d, d2h, duplex, with_compute)
+            if score < _PROBE_PASS_RATIO or tried >= _PROBE_MAX_CANDIDATES:
+                break
+            # replace the stream that waited; a fresh stream from torch's pool
+            # lands on the least-used hardware queue
+            if up_c >= _PROBE_PASS_RATIO:
+                h2d = torch.cuda.Stream(device)
+            else:  # d2h shares with the compute stream or with h2d
+                d2h = torch.cuda.Stream(device)
+            tried += 1
+        torch.cuda.synchronize(device)
+    score, h2d, d2h, duplex, with_compute = best
+    report = {"duplex_ratio": round(duplex, 3), "with_compute_ratio": round(with_compute, 3),
+              "streams_tried": tried, "concurrent": score < _PROBE_PASS_RATIO}
+    if not report["concurrent"]:
+        warnings.warn(
+            f"OffloadAdam: no pair of side streams ran copies concurrently ({report}); the "
+            "streaming step will be slower.  Export GPU_MAX_HW_QUEUES=8 before starting Python.",
+            stacklevel=3,
+        )
+    return h2d, d2h, report
 
 
 def _copy_by_kernel(dst, src, stream, workgroups=None):
@@ -189,10 +293,18 @@ class OffloadAdam(Optimizer):
         self.device_states = {}
         self.h2d_events = {}
         self.d2h_events = {}
-        self.h2d_stream = torch.cuda.Stream()
-        self.d2h_stream = self.h2d_stream if _ONE_TRANSFER_STREAM else torch.cuda.Stream()
+        self.transfer_stream_report = None
         if self._offload_params:
             self._check_copy_engines()
+        if self._offload_params and _PROBE_TRANSFER_STREAMS and not _ONE_TRANSFER_STREAM:
+            self.h2d_stream, self.d2h_stream, self.transfer_stream_report = pick_transfer_streams(
+                self._offload_params[0].device
+            )
+            if self.verbose > 0:
+                print(f"Transfer streams: {self.transfer_stream_report}")
+        else:
+            self.h2d_stream = torch.cuda.Stream()
+            self.d2h_stream = self.h2d_stream if _ONE_TRANSFER_STREAM else torch.cuda.Stream()
         self._param2group = {p: g for g in self.param_groups for p in g["params"]}
         # first module in forward order that owns each offloaded param ('lazy' policy)
         self._prefetch_module = {}

@@ -456,3 +456,23 @@ def test_adam_state_dict_round_trip_keeps_fp32_master():
         assert opt2.state[p2]["master_params"].dtype == torch.float32
         assert torch.equal(opt.state[p]["master_params"], opt2.state[p2]["master_params"])
         assert opt2.state[p2]["step"] == 1
+
+
+def test_transfer_streams_are_picked_by_measured_concurrency():
+    """With more live streams than hardware queues, the optimizer still ends up
+    with side streams whose copies run beside each other and beside kernels."""
+    from offload_adam_amd.offload_adam import pick_transfer_streams
+
+    crowd = [torch.cuda.Stream() for _ in range(5)]
+    for s in crowd:
+        with torch.cuda.stream(s):
+            torch.zeros(16, device="cuda")
+    torch.cuda.synchronize()
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")  # a failed search warns
+        h2d, d2h, report = pick_transfer_streams(torch.device("cuda:0"))
+    assert h2d.cuda_stream != d2h.cuda_stream
+    assert report["concurrent"] and report["duplex_ratio"] < 0.85, report
+    assert report["with_compute_ratio"] < 0.85, report
+    _, opt = run_offload_adam("stochastic_rounding", steps=1, ga=1)
+    assert opt.transfer_stream_report["concurrent"], opt.transfer_stream_report
