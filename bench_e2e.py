@@ -188,7 +188,9 @@ def link_bytes_per_step(opt, grad_accum):
     n = sum(p.numel() for p in opt._offload_params)
     state_b = sum(torch.empty(0, dtype=d).element_size()
                   for k, d in opt.offload_config.items() if k != "grad")
-    if opt._step_in_backward:
+    if not opt.offload_grads:
+        h2d = d2h = n * state_b
+    elif opt._step_in_backward:
         h2d = n * (2 * (grad_accum - 1) + state_b)
         d2h = n * (2 * (grad_accum - 1) + state_b)
     else:
@@ -207,7 +209,8 @@ def run(args):
     torch.cuda.set_device(dev)
     cfg = MODELS[args.model]
     out = {"model": args.model, "mode": args.mode, "seq": args.seq, "batch": 1,
-           "grad_accum": args.grad_accum, "max_grad_norm": args.max_grad_norm}
+           "grad_accum": args.grad_accum, "max_grad_norm": args.max_grad_norm,
+           "offload_grads": not args.grads_on_device}
 
     out["link_peak"] = measure_link()
 
@@ -245,7 +248,8 @@ def run(args):
         warnings.simplefilter("ignore")
         opt = OffloadAdam(model, lr=1e-5, mode=args.mode, max_grad_norm=args.max_grad_norm,
                           inplace_param_threshold=1024 * 1024, prefetch_policy="eager",
-                          decoupled_weight_decay=True)
+                          decoupled_weight_decay=True, offload_grads=not args.grads_on_device,
+                          prefetch_bytes=int(args.prefetch_gib * 2**30) if args.prefetch_gib else None)
     torch.cuda.synchronize()
     out["optimizer_init_s"] = round(time.perf_counter() - t0, 2)
     out["offloaded_params"] = len(opt._offload_params)
@@ -288,6 +292,8 @@ def main():
     ap.add_argument("--one-transfer-stream", action="store_true")
     ap.add_argument("--prefetch-gib", type=float, default=None,
                     help="device staging budget of the H2D prefetch window")
+    ap.add_argument("--grads-on-device", action="store_true",
+                    help="OffloadAdam(offload_grads=False): the gradient sum stays in HBM")
     ap.add_argument("--runtime-copy-engines", action="store_true",
                     help="leave the SDMA engine of each copy to the HIP runtime "
                          "(do not load the fixed-engine tools library)")
@@ -296,12 +302,10 @@ def main():
         import os
 
         os.environ["OFFLOAD_ADAM_COPY_ENGINES"] = "off"  # before the package is imported
-    if args.one_transfer_stream or args.prefetch_gib:
+    if args.one_transfer_stream:
         from offload_adam_amd import offload_adam as _oa_mod
 
         _oa_mod._ONE_TRANSFER_STREAM = args.one_transfer_stream
-        if args.prefetch_gib:
-            _oa_mod.OffloadAdam._PREFETCH_BYTES = int(args.prefetch_gib * 2**30)
     if args.d2h_workgroups:
         from offload_adam_amd import offload_adam as _oa_mod
 

@@ -476,3 +476,49 @@ def test_transfer_streams_are_picked_by_measured_concurrency():
     assert report["with_compute_ratio"] < 0.85, report
     _, opt = run_offload_adam("stochastic_rounding", steps=1, ga=1)
     assert opt.transfer_stream_report["concurrent"], opt.transfer_stream_report
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("ga", [1, 3])
+def test_grads_on_device_gives_identical_results(fixed_seed, mode, ga):
+    """offload_grads=False changes where the gradient sum waits, nothing else."""
+    ref_model, ref_opt = run_offload_adam(mode, steps=4, ga=ga, decoupled_weight_decay=True)
+    model, opt = run_offload_adam(mode, steps=4, ga=ga, decoupled_weight_decay=True,
+                                  offload_grads=False)
+    assert_same_params(ref_model, model)
+    for pr, p in zip(ref_model.parameters(), model.parameters()):
+        if p in opt._inplace_params:
+            continue
+        assert "grad" in ref_opt.state[pr] and ref_opt.state[pr]["grad"].is_pinned()
+        assert "grad" not in opt.state[p]  # no host gradient buffer at all
+        for key in opt._non_grad_keys:
+            a, b = ref_opt.state[pr][key], opt.state[p][key]
+            assert b.is_pinned() and torch.equal(a.view(torch.uint8), b.view(torch.uint8)), key
+    per_elem = {"stochastic_rounding": 4, "fp32_master": 8, "fp31_master": 6,
+                "fp32_master_custom_rounding": 6}[mode]
+    n = sum(p.numel() for p in opt._offload_params)
+    assert opt._estimate_pinned_bytes(opt._offload_params) == n * per_elem
+    assert ref_opt._estimate_pinned_bytes(ref_opt._offload_params) == n * (per_elem + 2)
+
+
+@pytest.mark.parametrize("ga", [1, 2])
+def test_grads_on_device_with_clipping(fixed_seed, ga):
+    ref_model, _ = run_offload_adam("fp31_master", steps=3, ga=ga, max_grad_norm=0.05)
+    model, opt = run_offload_adam("fp31_master", steps=3, ga=ga, max_grad_norm=0.05,
+                                  offload_grads=False)
+    assert float(opt._clip_coef) < 1.0
+    assert_same_params(ref_model, model)
+
+
+@pytest.mark.parametrize("prefetch_bytes", [0, 200_000, 1 << 30])
+def test_prefetch_budget_does_not_change_results(fixed_seed, prefetch_bytes):
+    """Window sizes from 'minimum two parameters' to 'everything staged after
+    the previous step' give the same bits."""
+    ref_model, _ = run_reference_adam("stochastic_rounding", steps=4, ga=3)
+    model, opt = run_offload_adam("stochastic_rounding", steps=4, ga=3,
+                                  prefetch_bytes=prefetch_bytes)
+    assert opt._PREFETCH_BYTES == prefetch_bytes
+    assert_same_params(ref_model, model)
+    model2, _ = run_offload_adam("stochastic_rounding", steps=4, ga=3,
+                                 prefetch_bytes=prefetch_bytes, offload_grads=False)
+    assert_same_params(ref_model, model2)
