@@ -1,0 +1,187 @@
+#!/usr/bin/env python3
+"""Per-kernel throughput of everything on the optimizer path besides the fused
+AdamW launch that ``bench.py`` measures: gradient L2 norm, clip coefficient,
+the fused AdamW kernel with the clip coefficient folded in (fp31_master), and
+the eight weight codecs.  One JSON line per kernel.
+
+    python bench_kernels.py [--reps 20] [--only norm,clip,adam,codecs]
+
+Shapes: the offloaded parameters of a Llama-3-8B-shaped decoder for the norm
+and AdamW kernels, one 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
+x10 for the codecs.  Every launch works on buffers that were not touched by the
+previous launches of the same kernel (the inputs rotate through more distinct
+buffers than the 256 MiB memory-side cache holds), so the figures are HBM
+figures.  ``achieved`` = algorithmic bytes of one launch / its duration between
+two HIP events on the launch stream; ``frac`` is against 8 TB/s.
+"""
+
+import argparse
+import json
+import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+ROWS, COLS = 4096, 14336
+
+
+def timed(fn, reps, torch):
+    """fn(i) launches once on rotation slot i; returns average microseconds."""
+    for i in range(3):
+        fn(i)
+    torch.cuda.synchronize()
+    evs = []
+    for i in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn(i)
+        b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in evs) / reps * 1e3
+
+
+def line(kernel, workload, alg_bytes, us, **extra):
+    gbs = alg_bytes / us / 1e3
+    out = {"kernel": kernel, "workload": workload, "alg_bytes_per_launch": int(alg_bytes),
+           "avg_launch_us": round(us, 2), "achieved_GBps": round(gbs, 1),
+           "peak_GBps": HBM_PEAK_GBS, "frac": round(gbs / HBM_PEAK_GBS, 4), "bound": "hbm"}
+    out.update(extra)
+    print(json.dumps(out), flush=True)
+
+
+def outlier_weight(torch, seed, dtype):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    w = torch.randn(ROWS, COLS, device="cuda", generator=g) * 0.02
+    mask = torch.rand(ROWS, COLS, device="cuda", generator=g) < 0.01
+    return torch.where(mask, w * 10, w).to(dtype)
+
+
+def bench_norm_and_clip(args, torch):
+    from offload_adam_amd import grad_clip
+
+    n_big = COLS * 4096
+    slots = 8  # 8 x 117 MB = 0.94 GB rotation
+    grads = [torch.randn(n_big, device="cuda", dtype=torch.bfloat16) * 5e-3 for _ in range(slots)]
+    norms = torch.zeros(slots, dtype=torch.bfloat16, device="cuda")
+    us = timed(lambda i: grad_clip.grad_norm_(grads[i % slots], norms[i % slots]), args.reps, torch)
+    line("grad_norm_partial_kernel + grad_norm_final_kernel", "bf16 gradient 14336x4096", 2 * n_big, us)
+    small = torch.randn(4096 * 1024, device="cuda", dtype=torch.bfloat16)
+    us = timed(lambda i: grad_clip.grad_norm_(small, norms[0]), args.reps, torch)
+    line("grad_norm_partial_kernel + grad_norm_final_kernel", "bf16 gradient 1024x4096 (cache resident)", 2 * small.numel(), us)
+    per_param = torch.rand(291, device="cuda").to(torch.bfloat16)
+    coef = torch.ones((), dtype=torch.bfloat16, device="cuda")
+    us = timed(lambda i: grad_clip.clip_coef_(per_param, 1.0, coef), args.reps, torch)
+    line("clip_coef_kernel", "291 per-parameter norms", 2 * 291, us, bound="latency")
+
+
+def bench_adam_clip(args, torch):
+    from offload_adam_amd.kernels import adam_step_fp31_master, adam_step_stochastic_rounding
+
+    n = COLS * 4096
+    slots = 4
+    clip = torch.tensor(0.3359375, dtype=torch.bfloat16, device="cuda")
+
+    def states(extra):
+        st = {"grad": torch.randn(n, device="cuda", dtype=torch.bfloat16) * 5e-3,
+              "exp_avg": torch.randn(n, device="cuda", dtype=torch.bfloat16) * 1e-4,
+              "exp_avg_sq": (torch.randn(n, device="cuda") * 1e-3).square().to(torch.bfloat16)}
+        if extra:
+            st["rounding_error"] = torch.zeros(n, dtype=torch.int16, device="cuda")
+        return st
+
+    ps = [torch.randn(n, device="cuda", dtype=torch.bfloat16) * 0.02 for _ in range(slots)]
+    st31 = [states(True) for _ in range(slots)]
+    us = timed(lambda i: adam_step_fp31_master(ps[i % slots], st31[i % slots], 1e-4, 0.01, 0.9,
+                                               0.999, 1e-8, 10, decoupled_weight_decay=True,
+                                               clip_coef=clip), args.reps, torch)
+    line("adam_vec_kernel<fp31_master, clip>", "one 14336x4096 parameter (hook-path launch)",
+         18 * n, us)
+    us = timed(lambda i: adam_step_stochastic_rounding(ps[i % slots], st31[i % slots], 1e-4, 0.01,
+                                                       0.9, 0.999, 1e-8, 10,
+                                                       decoupled_weight_decay=True),
+               args.reps, torch)
+    line("adam_vec_kernel<stochastic_rounding>", "one 14336x4096 parameter (hook-path launch)",
+         14 * n, us)
+
+
+def bench_codecs(args, torch):
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    n = ROWS * COLS
+    slots = 6
+    bf16 = torch.bfloat16
+    ws = [outlier_weight(torch, s, bf16) for s in range(slots)]
+    wl = "4096x14336 bf16 weight"
+
+    q8 = [torch.empty(ROWS, COLS, dtype=torch.int8, device="cuda") for _ in range(slots)]
+    s8 = [torch.empty(ROWS, dtype=bf16, device="cuda") for _ in range(slots)]
+    us = timed(lambda i: ops.quantize_int8_into(ws[i % slots], q8[i % slots], s8[i % slots]),
+               args.reps, torch)
+    line("quant_int8_kernel", wl, n * 3 + ROWS * 2, us)
+    us = timed(lambda i: ops.dequantize_int8(q8[i % slots], s8[i % slots], bf16), args.reps, torch)
+    line("dequant_int8_kernel", wl, n * 3 + ROWS * 2, us)
+
+    g = 128
+    q4 = [torch.empty(COLS // 8, ROWS, dtype=torch.int32, device="cuda") for _ in range(slots)]
+    s4 = [torch.empty(COLS // g, ROWS, dtype=bf16, device="cuda") for _ in range(slots)]
+    us = timed(lambda i: ops.quantize_int4_into(ws[i % slots], g, q4[i % slots], s4[i % slots]),
+               args.reps, torch)
+    line("quant_int4_kernel", wl + ", group 128", n * 2.5 + n // g * 2, us)
+    us = timed(lambda i: ops.dequantize_int4(q4[i % slots], s4[i % slots], g, bf16),
+               args.reps, torch)
+    line("dequant_int4_kernel", wl + ", group 128", n * 2.5 + n // g * 2, us)
+
+    b = 64
+    qn = [torch.empty(ROWS, COLS // 2, dtype=torch.uint8, device="cuda") for _ in range(slots)]
+    an = [torch.empty(ROWS * (COLS // b), dtype=torch.float32, device="cuda")
+          for _ in range(slots)]
+    us = timed(lambda i: ops.quantize_nf4_into(ws[i % slots], b, qn[i % slots], an[i % slots]),
+               args.reps, torch)
+    line("quant_nf4_kernel", wl + ", block 64", n * 2.5 + n // b * 4, us)
+    us = timed(lambda i: ops.dequantize_nf4(qn[i % slots], an[i % slots], COLS, b, bf16),
+               args.reps, torch)
+    line("dequant_nf4_kernel", wl + ", block 64", n * 2.5 + n // b * 4, us)
+
+    qf = [torch.empty(ROWS, COLS // 2, dtype=torch.uint8, device="cuda") for _ in range(slots)]
+    sf = [torch.empty(ROWS, COLS // 16, dtype=torch.float8_e4m3fn, device="cuda")
+          for _ in range(slots)]
+    gf = [torch.zeros((), dtype=torch.float32, device="cuda") for _ in range(slots)]
+    us = timed(lambda i: ops.quantize_nvfp4_into(ws[i % slots], qf[i % slots], sf[i % slots],
+                                                 gf[i % slots]), args.reps, torch)
+    line("nvfp4_amax_partial_kernel + nvfp4_global_scale_kernel + quant_nvfp4_kernel", wl + ", group 16",
+         n * 2 + n * 2.5 + n // 16, us,
+         note="three launches: per-block amax (reads the weight), global scale, encode (reads it again)")
+    us = timed(lambda i: ops.dequantize_nvfp4(qf[i % slots], sf[i % slots], gf[i % slots], COLS,
+                                              bf16), args.reps, torch)
+    line("dequant_nvfp4_kernel", wl + ", group 16", n * 2.5 + n // 16, us)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--only", default="norm,adam,codecs")
+    args = ap.parse_args()
+
+    import torch
+
+    from offload_adam_amd import _lib
+
+    if not torch.cuda.is_available():
+        print("bench_kernels.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _lib.load()
+    torch.cuda.set_device(0)
+    todo = set(args.only.split(","))
+    if "norm" in todo:
+        bench_norm_and_clip(args, torch)
+    if "adam" in todo:
+        bench_adam_clip(args, torch)
+    if "codecs" in todo:
+        bench_codecs(args, torch)
+
+
+if __name__ == "__main__":
+    main()

@@ -167,10 +167,11 @@ int oa_adam_multi(int mode, int count, void* const* params, const void* const* g
  * B. Gradient L2 norm per parameter and the global clip coefficient.
  * ---------------------------------------------------------------------- */
 
-/* Bytes of device scratch oa_grad_norm_bf16 needs.  The caller allocates it
- * (64-byte aligned), zero-fills it ONCE, and may reuse it for every later call
- * on the same stream: each launch leaves it zeroed again.  Launches that may
- * overlap (different streams) need separate workspaces. */
+/* Bytes of device scratch oa_grad_norm_bf16 and oa_quant_nvfp4 need (per-block
+ * partial results between their two launches).  The caller allocates it
+ * (64-byte aligned) and may reuse it for every later call on the same stream;
+ * its contents need no initialisation.  Launches that may overlap (different
+ * streams) need separate workspaces. */
 size_t oa_norm_workspace_bytes(void);
 
 /* Replaces `torch.norm(grad, 2.0)` on the accumulated bf16 gradient
@@ -254,12 +255,12 @@ int oa_dequant_nf4(const void* packed, const void* absmax, int64_t rows,
 /* NVFP4: e2m1 codes in blocks of 16 with float8_e4m3fn block scales and one
  * fp32 tensor scale.  Replaces _quantize_nvfp4_triton
  * (src/offload_adam/qweight/nvfp4.py:660-732; spec: quantize_nvfp4_blockwise +
- * pack_fp4, nvfp4.py:72-81, 133-173).  Two launches: tensor amax, then encode.
+ * pack_fp4, nvfp4.py:72-81, 133-173).  Three launches: per-block amax, global
+ * scale, encode.
  *   packed        uint8[rows * cols/2], even column in the LOW nibble
  *   block_scale   uint8[rows * cols/16], float8_e4m3fn bit patterns
  *   global_scale  ONE f32 (device), written: max(amax,1e-12) / (448*6)
- *   workspace     as for oa_grad_norm_bf16 (oa_norm_workspace_bytes() bytes,
- *                 zero-filled once)
+ *   workspace     as for oa_grad_norm_bf16 (oa_norm_workspace_bytes() bytes)
  * cols % 16 == 0. */
 int oa_quant_nvfp4(const void* src, int src_dtype, int64_t src_row_stride,
                    int64_t rows, int64_t cols, void* packed, void* block_scale,

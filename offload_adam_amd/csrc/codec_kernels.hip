@@ -501,29 +501,41 @@ __device__ __forceinline__ float e2m1_value(uint32_t code) {
   return __uint_as_float(((code & 8u) << 28) | mag);
 }
 
-struct AmaxWorkspace {  // same footprint as the norm workspace
-  unsigned int ticket;
-  unsigned int pad[15];
-  float partial[1024];
-};
+constexpr int kAmaxMaxBlocks = 16384;  // floats of the shared norm/amax workspace
+constexpr int kAmaxUnroll = 4;         // octets in flight per lane
 
-// Tensor-wide max |x| -> global scale = max(amax, 1e-12) / (448 * 6).
+// Tensor-wide max |x|, first launch: one partial maximum per block.  Octets of a
+// row-contiguous matrix are addressed flat (no per-octet division).
 template <int SRC>
 __global__ void __launch_bounds__(kT)
-nvfp4_global_scale_kernel(const void* __restrict__ src, int64_t stride, int64_t rows,
-                          int64_t cols, int vec, float* __restrict__ gs_out,
-                          AmaxWorkspace* __restrict__ ws) {
+nvfp4_amax_partial_kernel(const void* __restrict__ src, int64_t stride, int64_t rows,
+                          int64_t cols, int vec, float* __restrict__ partial) {
   __shared__ float lds[kT / kWave];
-  __shared__ bool is_last;
   float a = 0.0f;
   const int64_t step = (int64_t)gridDim.x * kT;
   if (vec) {
     const int64_t opr = cols >> 3, total = rows * opr;
-    for (int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x; o < total; o += step) {
-      const int64_t row = o / opr, c8 = o - row * opr;
-      float x[8];
-      load8<SRC>(src, row * stride + c8 * 8, x);
-      a = fmaxf(a, absmax8(x));
+    const bool flat = stride == cols;
+    int64_t o = (int64_t)blockIdx.x * kT * kAmaxUnroll + threadIdx.x;
+    for (; o < total; o += step * kAmaxUnroll) {
+      float x[kAmaxUnroll][8];
+#pragma unroll
+      for (int k = 0; k < kAmaxUnroll; ++k) {
+        const int64_t ok = o + (int64_t)k * kT;
+        if (ok < total) {
+          int64_t at = ok * 8;
+          if (!flat) {
+            const int64_t row = ok / opr;
+            at = row * stride + (ok - row * opr) * 8;
+          }
+          load8<SRC>(src, at, x[k]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) x[k][j] = 0.0f;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kAmaxUnroll; ++k) a = fmaxf(a, absmax8(x[k]));
     }
   } else {
     const int64_t total = rows * cols;
@@ -533,22 +545,18 @@ nvfp4_global_scale_kernel(const void* __restrict__ src, int64_t stride, int64_t 
     }
   }
   const float m = block_max(a, lds);
-  if (threadIdx.x == 0) {
-    __hip_atomic_store(&ws->partial[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();
-    is_last = (atomicAdd(&ws->ticket, 1u) == gridDim.x - 1);
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
+  if (threadIdx.x == 0) partial[blockIdx.x] = m;
+}
+
+// Second launch: global scale = max(amax, 1e-12) / (448 * 6).
+__global__ void __launch_bounds__(kT)
+nvfp4_global_scale_kernel(const float* __restrict__ partial, int blocks,
+                          float* __restrict__ gs_out) {
+  __shared__ float lds[kT / kWave];
   float t = 0.0f;
-  for (unsigned int b = threadIdx.x; b < gridDim.x; b += kT)
-    t = fmaxf(t, __hip_atomic_load(&ws->partial[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  for (int b = threadIdx.x; b < blocks; b += kT) t = fmaxf(t, partial[b]);
   t = block_max(t, lds);
-  if (threadIdx.x == 0) {
-    *gs_out = fmaxf(t, kEps) / (448.0f * 6.0f);
-    __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (threadIdx.x == 0) *gs_out = fmaxf(t, kEps) / (448.0f * 6.0f);
 }
 
 __device__ __forceinline__ uint32_t nvfp4_pack8(const float (&x)[8], float inv_eff) {
@@ -862,15 +870,20 @@ extern "C" int oa_quant_nvfp4(const void* src, int src_dtype, int64_t src_row_st
   if (rows * cols > 0 && (!packed || !block_scale)) return OA_EINVAL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int vec = rows_vec(src, src_dtype, src_row_stride, cols);
+  const int64_t per_block = (int64_t)kT * (vec ? kAmaxUnroll : 8);
   const int64_t work = vec ? rows * (cols / 8) : rows * cols;
-  int64_t rblocks = (work + (int64_t)kT * 8 - 1) / ((int64_t)kT * 8);
+  int64_t rblocks = (work + per_block - 1) / per_block;
   if (rblocks < 1) rblocks = 1;
-  if (rblocks > 1024) rblocks = 1024;
+  if (rblocks > kAmaxMaxBlocks) rblocks = kAmaxMaxBlocks;
+  float* partial = static_cast<float*>(workspace);
   OA_DISPATCH_DT(src_dtype,
-                 hipLaunchKernelGGL(nvfp4_global_scale_kernel<DT>, dim3((unsigned)rblocks),
+                 hipLaunchKernelGGL(nvfp4_amax_partial_kernel<DT>, dim3((unsigned)rblocks),
                                     dim3(kT), 0, s, src, src_row_stride, rows, cols, vec,
-                                    static_cast<float*>(global_scale),
-                                    static_cast<AmaxWorkspace*>(workspace)));
+                                    partial));
+  rc = launch_status();
+  if (rc) return rc;
+  hipLaunchKernelGGL(nvfp4_global_scale_kernel, dim3(1), dim3(kT), 0, s, partial, (int)rblocks,
+                     static_cast<float*>(global_scale));
   rc = launch_status();
   if (rc || rows * cols == 0) return rc;
   if (vec && aligned_to(packed, 4) && aligned_to(block_scale, 4)) {
