@@ -5,11 +5,14 @@ shared object has not been built, every operator raises.
 """
 
 import ctypes
+import os
 import threading
 from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint64, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "liboffload_adam_hip.so"
+# OFFLOAD_ADAM_HIP_LIB points at another build of the same library (kernel tuning).
+LIB_PATH = Path(os.environ.get("OFFLOAD_ADAM_HIP_LIB")
+                or Path(__file__).resolve().parent / "liboffload_adam_hip.so")
 
 OA_RNG_TRITON = 0
 OA_RNG_X8 = 1

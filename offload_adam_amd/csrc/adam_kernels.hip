@@ -293,10 +293,38 @@ __device__ __forceinline__ void adam_tile(const AdamArgs& a, int64_t tile, bool 
   }
 }
 
+// Workgroup -> tile.  The dispatcher deals consecutive workgroups to the 8 XCDs
+// round-robin (workgroup b runs on XCD b % 8), each with its own L2.  With
+// tile = b every XCD touches every 8th tile of every array; mapping so that an
+// XCD owns runs of OA_ADAM_XCD_CHUNK consecutive tiles gives each L2 and the
+// memory channels behind it longer sequential streams (measured on a 4-read /
+// 3-write stream kernel of this shape: +3 % at 15 GB, +10 % at 0.8 GB per
+// launch).  The map is a bijection on [0, round_up(tiles, 8 * chunk)); grids are
+// padded to that size and surplus workgroups exit.
+#ifndef OA_ADAM_XCD_CHUNK
+#define OA_ADAM_XCD_CHUNK 64
+#endif
+constexpr uint32_t kXcds = 8;
+constexpr uint32_t kXcdChunk = OA_ADAM_XCD_CHUNK;
+
+__device__ __forceinline__ uint32_t xcd_tile(uint32_t b) {
+  if (kXcdChunk == 0) return b;
+  const uint32_t x = b % kXcds, j = b / kXcds;
+  const uint32_t c = j / kXcdChunk, r = j % kXcdChunk;
+  return (c * kXcds + x) * kXcdChunk + r;
+}
+inline uint32_t xcd_grid(uint32_t tiles) {
+  if (kXcdChunk == 0) return tiles;
+  const uint32_t q = kXcds * kXcdChunk;
+  return (tiles + q - 1) / q * q;
+}
+
 template <int MODE, bool DEC, bool CLIP, int RNG>
 __global__ void __launch_bounds__(OA_ADAM_THREADS)
-adam_vec_kernel(const AdamArgs a) {
-  adam_tile<MODE, DEC, CLIP, RNG>(a, blockIdx.x, blockIdx.x == gridDim.x - 1);
+adam_vec_kernel(const AdamArgs a, uint32_t tiles) {
+  const uint32_t tile = xcd_tile(blockIdx.x);
+  if (tile >= tiles) return;
+  adam_tile<MODE, DEC, CLIP, RNG>(a, tile, tile == tiles - 1);
 }
 
 // Multi-tensor form: one launch covers up to kMultiMax parameters.  The
@@ -325,8 +353,10 @@ struct MultiArgs {
 template <int MODE, bool DEC, bool CLIP, int RNG>
 __global__ void __launch_bounds__(OA_ADAM_THREADS)
 adam_multi_kernel(const MultiArgs ma) {
+  const uint32_t b = xcd_tile(blockIdx.x);
+  if (b >= ma.tile_start[ma.count]) return;
   int t = 0;
-  while (t + 1 < ma.count && blockIdx.x >= ma.tile_start[t + 1]) ++t;
+  while (t + 1 < ma.count && b >= ma.tile_start[t + 1]) ++t;
   AdamArgs a;
   a.p = ma.p[t];
   a.g = ma.g[t];
@@ -344,8 +374,8 @@ adam_multi_kernel(const MultiArgs ma) {
   a.eps = ma.eps;
   a.k0 = ma.k0[t];
   a.k1 = ma.k1[t];
-  const uint32_t tile = blockIdx.x - ma.tile_start[t];
-  adam_tile<MODE, DEC, CLIP, RNG>(a, tile, blockIdx.x + 1 == ma.tile_start[t + 1]);
+  const uint32_t tile = b - ma.tile_start[t];
+  adam_tile<MODE, DEC, CLIP, RNG>(a, tile, b + 1 == ma.tile_start[t + 1]);
 }
 
 template <int MODE, bool DEC, bool CLIP, int RNG>
@@ -354,9 +384,9 @@ int launch(const AdamArgs& a, bool vec, hipStream_t s) {
   if (vec) {
     const int64_t per_block = (int64_t)T * OA_ADAM_UNROLL * 8;
     int64_t blocks = (a.n + per_block - 1) / per_block;
-    if (blocks > 0x7FFFFFFFll) return OA_ERANGE;
-    hipLaunchKernelGGL((adam_vec_kernel<MODE, DEC, CLIP, RNG>), dim3((unsigned)blocks),
-                       dim3(T), 0, s, a);
+    if (blocks > 0x7FFF0000ll) return OA_ERANGE;
+    hipLaunchKernelGGL((adam_vec_kernel<MODE, DEC, CLIP, RNG>),
+                       dim3(xcd_grid((uint32_t)blocks)), dim3(T), 0, s, a, (uint32_t)blocks);
   } else {
     int64_t blocks = (a.n + T - 1) / T;
     if (blocks > 65536) blocks = 65536;  // grid-stride beyond this
@@ -524,7 +554,7 @@ template <int MODE, int RNG>
 int launch_multi(const MultiArgs& ma, bool dec, unsigned tiles, hipStream_t s) {
   const bool clip = ma.clip != nullptr;
 #define OA_LAUNCH_MULTI(D, C)                                                            \
-  hipLaunchKernelGGL((adam_multi_kernel<MODE, D, C, RNG>), dim3(tiles),                   \
+  hipLaunchKernelGGL((adam_multi_kernel<MODE, D, C, RNG>), dim3(xcd_grid(tiles)),         \
                      dim3(OA_ADAM_THREADS), 0, s, ma)
   if (dec) {
     if (clip) OA_LAUNCH_MULTI(true, true); else OA_LAUNCH_MULTI(true, false);
@@ -630,8 +660,8 @@ extern "C" int oa_adam_multi(int mode, int count, void* const* params,
       continue;
     }
     int64_t t_tiles = (n + kPerTile - 1) / kPerTile;
-    if (t_tiles > 0x7FFFFFFFll) return OA_ERANGE;
-    if (ma.count == kMultiMax || tiles + (uint64_t)t_tiles > 0x7FFFFFFFull) {
+    if (t_tiles > 0x7FFF0000ll) return OA_ERANGE;
+    if (ma.count == kMultiMax || tiles + (uint64_t)t_tiles > 0x7FFF0000ull) {
       int rc = flush();
       if (rc) return rc;
     }

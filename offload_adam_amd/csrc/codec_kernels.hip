@@ -128,6 +128,24 @@ __device__ __forceinline__ float block_max(float x, float* lds) {
   return t;
 }
 
+// The flat kernels give every lane kOct octets, kT lanes apart, all loaded
+// before the first is used.
+constexpr int kOct = 4;
+
+// How octet index o maps to an element offset: rows stored back to back need no
+// row index at all; otherwise row = o / octets_per_row, in 32 bits when it fits.
+enum { kFlat = 0, kDiv32 = 1, kDiv64 = 2 };
+
+__device__ __forceinline__ int64_t octet_row(int64_t o, int64_t opr, int mode) {
+  if (mode == kDiv64) return o / opr;
+  return (int64_t)((uint32_t)o / (uint32_t)opr);
+}
+__device__ __forceinline__ int64_t octet_elem(int64_t o, int64_t opr, int64_t stride, int mode) {
+  if (mode == kFlat) return o * 8;
+  const int64_t row = octet_row(o, opr, mode);
+  return row * stride + (o - row * opr) * 8;
+}
+
 // ------------------------------------------------------------------- int8
 
 __device__ __forceinline__ int32_t q_int8(float x, float inv) {
@@ -136,8 +154,12 @@ __device__ __forceinline__ int32_t q_int8(float x, float inv) {
   return (int32_t)t;
 }
 
-// One block per row: pass 1 folds |x| into the row maximum, pass 2 re-reads the
-// row (L2-resident: a row is tens of KiB) and writes the codes.
+constexpr int kRowCache = 8;  // octets a lane keeps in registers between the two passes
+
+// One block per row.  Pass 1 loads the row (all of a lane's octets in flight at
+// once, kept in registers when the row has at most kT * kRowCache octets) and
+// folds |x| into the row maximum; pass 2 encodes from the registers.  Longer rows
+// are re-read in pass 2 (L2-resident: a row is tens of KiB).
 template <int SRC>
 __global__ void __launch_bounds__(kT)
 quant_int8_kernel(const void* __restrict__ src, int64_t stride, int64_t cols,
@@ -146,11 +168,28 @@ quant_int8_kernel(const void* __restrict__ src, int64_t stride, int64_t cols,
   const int64_t row = blockIdx.x;
   const int64_t base = row * stride;
   const int64_t octets = vec ? cols >> 3 : 0;
+  const bool cached = octets <= (int64_t)kT * kRowCache;
+  float xc[kRowCache][8];
   float a = 0.0f;
-  for (int64_t o = threadIdx.x; o < octets; o += kT) {
-    float x[8];
-    load8<SRC>(src, base + o * 8, x);
-    a = fmaxf(a, absmax8(x));
+  if (cached) {
+#pragma unroll
+    for (int k = 0; k < kRowCache; ++k) {
+      const int64_t o = threadIdx.x + (int64_t)k * kT;
+      if (o < octets) {
+        load8<SRC>(src, base + o * 8, xc[k]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xc[k][j] = 0.0f;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kRowCache; ++k) a = fmaxf(a, absmax8(xc[k]));
+  } else {
+    for (int64_t o = threadIdx.x; o < octets; o += kT) {
+      float x[8];
+      load8<SRC>(src, base + o * 8, x);
+      a = fmaxf(a, absmax8(x));
+    }
   }
   for (int64_t c = octets * 8 + threadIdx.x; c < cols; c += kT)
     a = fmaxf(a, fabsf(load1<SRC>(src, base + c)));
@@ -160,9 +199,7 @@ quant_int8_kernel(const void* __restrict__ src, int64_t stride, int64_t cols,
   if (threadIdx.x == 0) store_scale(scales, sdt, row, scale);
 
   int8_t* qr = q + row * cols;
-  for (int64_t o = threadIdx.x; o < octets; o += kT) {
-    float x[8];
-    load8<SRC>(src, base + o * 8, x);
+  auto encode = [&](const float (&x)[8], int64_t o) {
     uint32_t w0 = 0, w1 = 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -170,6 +207,19 @@ quant_int8_kernel(const void* __restrict__ src, int64_t stride, int64_t cols,
       w1 |= ((uint32_t)q_int8(x[4 + k], inv) & 0xFFu) << (8 * k);
     }
     *reinterpret_cast<u32x2*>(qr + o * 8) = u32x2{w0, w1};
+  };
+  if (cached) {
+#pragma unroll
+    for (int k = 0; k < kRowCache; ++k) {
+      const int64_t o = threadIdx.x + (int64_t)k * kT;
+      if (o < octets) encode(xc[k], o);
+    }
+  } else {
+    for (int64_t o = threadIdx.x; o < octets; o += kT) {
+      float x[8];
+      load8<SRC>(src, base + o * 8, x);
+      encode(x, o);
+    }
   }
   for (int64_t c = octets * 8 + threadIdx.x; c < cols; c += kT)
     qr[c] = (int8_t)q_int8(load1<SRC>(src, base + c), inv);
@@ -179,21 +229,37 @@ template <int OUT>
 __global__ void __launch_bounds__(kT)
 dequant_int8_kernel(const int8_t* __restrict__ q, const void* __restrict__ scales, int sdt,
                     int64_t rows, int64_t cols, void* __restrict__ out, int64_t ostride,
-                    int vec) {
+                    int vec, int mode) {
   if (vec) {
-    const int64_t opr = cols >> 3;
-    const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
-    if (o >= rows * opr) return;
-    const int64_t row = o / opr, c8 = o - row * opr;
-    const float s = load_scale(scales, sdt, row);
-    const u32x2 w = *reinterpret_cast<const u32x2*>(q + row * cols + c8 * 8);
-    float y[8];
+    const int64_t opr = cols >> 3, total = rows * opr;
+    const int64_t o0 = (int64_t)blockIdx.x * (kT * kOct) + threadIdx.x;
+    u32x2 w[kOct];
+    float s[kOct];
+    int64_t at[kOct];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int32_t v = (int32_t)(int8_t)((w[k >> 2] >> (8 * (k & 3))) & 0xFFu);
-      y[k] = (float)v * s;
+    for (int k = 0; k < kOct; ++k) {
+      const int64_t o = o0 + (int64_t)k * kT;
+      w[k] = u32x2{0u, 0u};
+      s[k] = 0.0f;
+      at[k] = 0;
+      if (o < total) {
+        const int64_t row = octet_row(o, opr, mode), c8 = o - row * opr;
+        w[k] = *reinterpret_cast<const u32x2*>(q + row * cols + c8 * 8);
+        s[k] = load_scale(scales, sdt, row);
+        at[k] = row * ostride + c8 * 8;
+      }
     }
-    store8<OUT>(out, row * ostride + c8 * 8, y);
+#pragma unroll
+    for (int k = 0; k < kOct; ++k) {
+      if (o0 + (int64_t)k * kT >= total) continue;
+      float y[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int32_t v = (int32_t)(int8_t)((w[k][j >> 2] >> (8 * (j & 3))) & 0xFFu);
+        y[j] = (float)v * s[k];
+      }
+      store8<OUT>(out, at[k], y);
+    }
   } else {
     const int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x;
     if (i >= rows * cols) return;
@@ -345,13 +411,78 @@ __constant__ float kNf4Lut[16] = {
 // the fp32 bit patterns, so the count equals the first-minimum argmin over the
 // fp32 distances for every input (the neighbours are the only candidates: the
 // codebook spacing is >= 0.079, rounding error of a distance <= 6e-8).
+constexpr uint32_t kNf4T[15] = {
+    0xbf591cd8u, 0xbf1c5270u, 0xbeeb847fu, 0xbeadea76u, 0xbe703cecu,
+    0xbe0d38bbu, 0xbd3a7870u, 0x3d22fb00u, 0x3df64863u, 0x3e5067e1u,
+    0x3e9582d5u, 0x3ec753fau, 0x3f006d04u, 0x3f248db0u, 0x3f5c89dau};
+
+// Counting thresholds without walking them.  With m = 16 * n:
+// bucket(m) = trunc(m + 16) clamped to [0, 31] is monotone in n, and the
+// thresholds are further apart (>= 0.0805) than a bucket is wide (0.0625), so
+// every bucket holds at most one.  For n in bucket k the thresholds of lower
+// buckets are below n and those of higher buckets above; the bucket's own
+// threshold, if any, is compared directly:
+//     code(n) = below[k] + (m >= 16 * own[k]),      own = +inf if none
+// Scaling by 16 is exact in fp32, so x * (16 * inv) == 16 * fl(x * inv) and
+// m >= 16 * t  <=>  n >= t: the kernel never forms n itself.  The table is built
+// at compile time with the same fp32 addition the kernel uses, so bucket(16 t_i)
+// here and bucket(m) on the GPU agree bit for bit.  The 32 entries of 8 bytes
+// cover the 64 LDS banks exactly once: the lookup has no bank conflicts.
+constexpr int nf4_bucket(float m) {  // m = 16 n
+  const float f = m + 16.0f;
+  if (!(f > 0.0f)) return 0;
+  if (f >= 31.0f) return 31;
+  return (int)f;
+}
+struct Nf4Buckets {
+  uint32_t own16[32];  // fp32 bits of 16 * (threshold inside the bucket), +inf if none
+  uint32_t below[32];  // thresholds in lower buckets
+};
+constexpr Nf4Buckets make_nf4_buckets() {
+  Nf4Buckets t{};
+  for (int k = 0; k < 32; ++k) {
+    t.own16[k] = 0x7F800000u;
+    t.below[k] = 0;
+  }
+  for (int i = 0; i < 15; ++i) {
+    const float t16 = __builtin_bit_cast(float, kNf4T[i]) * 16.0f;
+    const int b = nf4_bucket(t16);
+    t.own16[b] = __builtin_bit_cast(uint32_t, t16);
+    for (int k = b + 1; k < 32; ++k) t.below[k] += 1;
+  }
+  return t;
+}
+constexpr bool nf4_buckets_distinct() {
+  int last = -1;
+  for (int i = 0; i < 15; ++i) {
+    const int b = nf4_bucket(__builtin_bit_cast(float, kNf4T[i]) * 16.0f);
+    if (b <= last) return false;
+    last = b;
+  }
+  return true;
+}
+static_assert(nf4_buckets_distinct(), "two NF4 thresholds share a bucket");
+__device__ const Nf4Buckets kNf4Buckets = make_nf4_buckets();
+
+__device__ __forceinline__ void nf4_buckets_to_lds(u32x2* lut) {
+  if (threadIdx.x < 32)
+    lut[threadIdx.x] = u32x2{kNf4Buckets.own16[threadIdx.x], kNf4Buckets.below[threadIdx.x]};
+}
+
+// m = 16 * (x / absmax); |m| <= 16 (1 + 2^-23) for finite input, so m + 16 lies in
+// (-1, 33) and the conversion to int is exact truncation.
+__device__ __forceinline__ uint32_t nf4_code16(float m, const u32x2* lut) {
+  int k = (int)(m + 16.0f);
+  k = k > 31 ? 31 : k;
+  k = k < 0 ? 0 : k;  // NaN
+  const u32x2 e = lut[k];
+  return e[1] + (uint32_t)(m >= __uint_as_float(e[0]));
+}
+
+// The same count by a four-level decision tree (no table): used by the generic
+// kernel, which has no block-wide prologue.
 #define NF4_T(i) __uint_as_float(kNf4T[i])
-__device__ __forceinline__ uint32_t nf4_code(float n) {
-  constexpr uint32_t kNf4T[15] = {
-      0xbf591cd8u, 0xbf1c5270u, 0xbeeb847fu, 0xbeadea76u, 0xbe703cecu,
-      0xbe0d38bbu, 0xbd3a7870u, 0x3d22fb00u, 0x3df64863u, 0x3e5067e1u,
-      0x3e9582d5u, 0x3ec753fau, 0x3f006d04u, 0x3f248db0u, 0x3f5c89dau};
-  // four-level decision tree over the sorted thresholds
+__device__ __forceinline__ uint32_t nf4_code_tree(float n) {
   const bool b3 = n >= NF4_T(7);
   const bool b2 = n >= (b3 ? NF4_T(11) : NF4_T(3));
   const bool b1 = n >= (b3 ? (b2 ? NF4_T(13) : NF4_T(9)) : (b2 ? NF4_T(5) : NF4_T(1)));
@@ -362,11 +493,13 @@ __device__ __forceinline__ uint32_t nf4_code(float n) {
 }
 #undef NF4_T
 
-__device__ __forceinline__ uint32_t nf4_pack8(const float (&x)[8], float inv) {
+// inv16 = 16 / absmax (the exact 16-fold of the reference's 1 / absmax)
+__device__ __forceinline__ uint32_t nf4_pack8(const float (&x)[8], float inv16, const u32x2* lut) {
   uint32_t w = 0;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const uint32_t hi = nf4_code(x[2 * j] * inv), lo = nf4_code(x[2 * j + 1] * inv);
+    const uint32_t hi = nf4_code16(x[2 * j] * inv16, lut);
+    const uint32_t lo = nf4_code16(x[2 * j + 1] * inv16, lut);
     w |= ((hi << 4) | lo) << (8 * j);
   }
   return w;
@@ -376,44 +509,67 @@ __device__ __forceinline__ uint32_t nf4_pack8(const float (&x)[8], float inv) {
 template <int SRC>
 __global__ void __launch_bounds__(kT)
 quant_nf4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
-                 int lpg, uint32_t* __restrict__ packed, float* __restrict__ absmax_out) {
-  const int64_t opr = cols >> 3;
-  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
-  const bool live = o < rows * opr;
-  float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  if (live) {
-    const int64_t row = o / opr, c8 = o - row * opr;
-    load8<SRC>(src, row * stride + c8 * 8, x);
+                 int lpg, int lpg_shift, uint32_t* __restrict__ packed,
+                 float* __restrict__ absmax_out, int mode) {
+  __shared__ u32x2 lut[32];
+  nf4_buckets_to_lds(lut);
+  const int64_t opr = cols >> 3, total = rows * opr;
+  const int64_t o0 = (int64_t)blockIdx.x * (kT * kOct) + threadIdx.x;
+  float x[kOct][8];
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    if (o < total) {
+      load8<SRC>(src, octet_elem(o, opr, stride, mode), x[k]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[k][j] = 0.0f;
+    }
   }
-  const float absmax = group_max(absmax8(x), lpg);
-  const float inv = 1.0f / fmaxf(absmax, kEps);
-  if (!live) return;
-  packed[o] = nf4_pack8(x, inv);
-  if ((threadIdx.x & (lpg - 1)) == 0) absmax_out[o / lpg] = absmax;
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    const float absmax = group_max(absmax8(x[k]), lpg);
+    const float inv16 = (1.0f / fmaxf(absmax, kEps)) * 16.0f;
+    if (o < total) {
+      packed[o] = nf4_pack8(x[k], inv16, lut);
+      if ((threadIdx.x & (lpg - 1)) == 0) absmax_out[o >> lpg_shift] = absmax;
+    }
+  }
 }
 
 template <int OUT>
 __global__ void __launch_bounds__(kT)
 dequant_nf4_kernel(const uint32_t* __restrict__ packed, const float* __restrict__ absmax,
-                   int64_t rows, int64_t cols, int lpg, void* __restrict__ out,
-                   int64_t ostride) {
+                   int64_t rows, int64_t cols, int lpg_shift, void* __restrict__ out,
+                   int64_t ostride, int mode) {
   __shared__ float lut[16];
   if (threadIdx.x < 16) lut[threadIdx.x] = kNf4Lut[threadIdx.x];
-  __syncthreads();
-  const int64_t opr = cols >> 3;
-  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
-  if (o >= rows * opr) return;
-  const int64_t row = o / opr, c8 = o - row * opr;
-  const uint32_t w = packed[o];
-  const float s = absmax[o / lpg];
-  float y[8];
+  const int64_t opr = cols >> 3, total = rows * opr;
+  const int64_t o0 = (int64_t)blockIdx.x * (kT * kOct) + threadIdx.x;
+  uint32_t w[kOct];
+  float s[kOct];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const uint32_t b = (w >> (8 * j)) & 0xFFu;
-    y[2 * j] = lut[b >> 4] * s;
-    y[2 * j + 1] = lut[b & 0xFu] * s;
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    w[k] = o < total ? packed[o] : 0u;
+    s[k] = o < total ? absmax[o >> lpg_shift] : 0.0f;
   }
-  store8<OUT>(out, row * ostride + c8 * 8, y);
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    if (o >= total) continue;
+    float y[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t b = (w[k] >> (8 * j)) & 0xFFu;
+      y[2 * j] = lut[b >> 4] * s[k];
+      y[2 * j + 1] = lut[b & 0xFu] * s[k];
+    }
+    store8<OUT>(out, octet_elem(o, opr, ostride, mode), y);
+  }
 }
 
 template <int SRC>
@@ -430,8 +586,8 @@ quant_nf4_generic(const void* __restrict__ src, int64_t stride, int64_t rows, in
   const float inv = 1.0f / fmaxf(a, kEps);
   absmax_out[t] = a;
   for (int64_t c = 0; c < block; c += 2) {
-    const uint32_t hi = nf4_code(load1<SRC>(src, base + c) * inv);
-    const uint32_t lo = nf4_code(load1<SRC>(src, base + c + 1) * inv);
+    const uint32_t hi = nf4_code_tree(load1<SRC>(src, base + c) * inv);
+    const uint32_t lo = nf4_code_tree(load1<SRC>(src, base + c + 1) * inv);
     packed[row * (cols / 2) + (gi * block + c) / 2] = (uint8_t)((hi << 4) | lo);
   }
 }
@@ -548,24 +704,48 @@ nvfp4_amax_partial_kernel(const void* __restrict__ src, int64_t stride, int64_t 
   if (threadIdx.x == 0) partial[blockIdx.x] = m;
 }
 
-// Second launch: global scale = max(amax, 1e-12) / (448 * 6).
-__global__ void __launch_bounds__(kT)
+// Second launch: global scale = max(amax, 1e-12) / (448 * 6).  One block of 1024
+// lanes, 4 partials per lane per trip, so 16384 partials are 4 dependent trips.
+constexpr int kScaleThreads = 1024;
+__global__ void __launch_bounds__(kScaleThreads)
 nvfp4_global_scale_kernel(const float* __restrict__ partial, int blocks,
                           float* __restrict__ gs_out) {
-  __shared__ float lds[kT / kWave];
+  __shared__ float lds[kScaleThreads / kWave];
   float t = 0.0f;
-  for (int b = threadIdx.x; b < blocks; b += kT) t = fmaxf(t, partial[b]);
-  t = block_max(t, lds);
-  if (threadIdx.x == 0) *gs_out = fmaxf(t, kEps) / (448.0f * 6.0f);
+  for (int b = threadIdx.x; b < blocks; b += 4 * kScaleThreads) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = b + k * kScaleThreads;
+      v[k] = i < blocks ? partial[i] : 0.0f;
+    }
+    t = fmaxf(fmaxf(t, fmaxf(v[0], v[1])), fmaxf(v[2], v[3]));
+  }
+  t = wave_max(t);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = t;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = lds[0];
+#pragma unroll
+    for (int w = 1; w < kScaleThreads / kWave; ++w) m = fmaxf(m, lds[w]);
+    *gs_out = fmaxf(m, kEps) / (448.0f * 6.0f);
+  }
 }
 
+// Eight e2m1 codes, even element in the low nibble.  gfx950 converts a pair of
+// fp32 values to packed FP4 in one instruction (v_cvt_scalef32_pk_fp4_f32 with a
+// scale of 1: round to nearest even on the e2m1 grid, saturating at 6, the sign
+// of zero kept) - bit for bit what e2m1_code() computes for every non-NaN input
+// (checked on the GPU over every float within 64 ulps of each grid point and
+// rounding boundary, a 1e-5 sweep of [-8, 8], denormals, infinities and
+// FLT_MAX).  A NaN becomes +-6 here and +-0 in e2m1_code(); a tensor with a NaN
+// has a NaN scale in the reference and is outside the codec's contract.
 __device__ __forceinline__ uint32_t nvfp4_pack8(const float (&x)[8], float inv_eff) {
   uint32_t w = 0;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const uint32_t lo = e2m1_code(x[2 * j] * inv_eff), hi = e2m1_code(x[2 * j + 1] * inv_eff);
-    w |= ((hi << 4) | lo) << (8 * j);
-  }
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[0] * inv_eff, x[1] * inv_eff, 1.0f, 0);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[2] * inv_eff, x[3] * inv_eff, 1.0f, 1);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[4] * inv_eff, x[5] * inv_eff, 1.0f, 2);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[6] * inv_eff, x[7] * inv_eff, 1.0f, 3);
   return w;
 }
 
@@ -580,32 +760,41 @@ template <int SRC>
 __global__ void __launch_bounds__(kT)
 quant_nvfp4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
                    uint32_t* __restrict__ packed, uint8_t* __restrict__ scale8,
-                   const float* __restrict__ gs_ptr) {
+                   const float* __restrict__ gs_ptr, int mode) {
   const int64_t opr = cols >> 3, total = rows * opr;
-  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
-  const bool live = o < total;
-  float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  if (live) {
-    const int64_t row = o / opr, c8 = o - row * opr;
-    load8<SRC>(src, row * stride + c8 * 8, x);
+  const int64_t o0 = (int64_t)blockIdx.x * (kT * kOct) + threadIdx.x;
+  float x[kOct][8];
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    if (o < total) {
+      load8<SRC>(src, octet_elem(o, opr, stride, mode), x[k]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[k][j] = 0.0f;
+    }
   }
   const float gs = *gs_ptr;
   const float inv_global = 1.0f / gs;
-  const float amax = group_max(absmax8(x), 2);
-  const uint32_t s8 = nvfp4_block_scale(amax, inv_global);
-  const float eff = e4m3fn_bits_to_f32(s8) * gs;
-  const float inv_eff = 1.0f / fmaxf(eff, kEps);
-  // gather the scales of the 4 blocks covered by 8 consecutive lanes
   const int lane = threadIdx.x & (kWave - 1), base = lane & ~7;
-  const uint32_t s4 = __shfl(s8, base, kWave) | (__shfl(s8, base + 2, kWave) << 8) |
-                      (__shfl(s8, base + 4, kWave) << 16) | (__shfl(s8, base + 6, kWave) << 24);
-  if (!live) return;
-  packed[o] = nvfp4_pack8(x, inv_eff);
-  const int64_t o_base = o - (lane & 7);
-  if (o_base + 8 <= total) {
-    if ((lane & 7) == 0) *reinterpret_cast<uint32_t*>(scale8 + (o_base >> 1)) = s4;
-  } else if ((lane & 1) == 0) {
-    scale8[o >> 1] = (uint8_t)s8;
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    const float amax = group_max(absmax8(x[k]), 2);
+    const uint32_t s8 = nvfp4_block_scale(amax, inv_global);
+    const float eff = e4m3fn_bits_to_f32(s8) * gs;
+    const float inv_eff = 1.0f / fmaxf(eff, kEps);
+    // gather the scales of the 4 blocks covered by 8 consecutive lanes
+    const uint32_t s4 = __shfl(s8, base, kWave) | (__shfl(s8, base + 2, kWave) << 8) |
+                        (__shfl(s8, base + 4, kWave) << 16) | (__shfl(s8, base + 6, kWave) << 24);
+    if (o >= total) continue;
+    packed[o] = nvfp4_pack8(x[k], inv_eff);
+    const int64_t o_base = o - (lane & 7);
+    if (o_base + 8 <= total) {
+      if ((lane & 7) == 0) *reinterpret_cast<uint32_t*>(scale8 + (o_base >> 1)) = s4;
+    } else if ((lane & 1) == 0) {
+      scale8[o >> 1] = (uint8_t)s8;
+    }
   }
 }
 
@@ -613,21 +802,31 @@ template <int OUT>
 __global__ void __launch_bounds__(kT)
 dequant_nvfp4_kernel(const uint32_t* __restrict__ packed, const uint8_t* __restrict__ scale8,
                      const float* __restrict__ gs_ptr, int64_t rows, int64_t cols,
-                     void* __restrict__ out, int64_t ostride) {
-  const int64_t opr = cols >> 3;
-  const int64_t o = (int64_t)blockIdx.x * kT + threadIdx.x;
-  if (o >= rows * opr) return;
-  const int64_t row = o / opr, c8 = o - row * opr;
-  const uint32_t w = packed[o];
-  const float eff = e4m3fn_bits_to_f32(scale8[o >> 1]) * (*gs_ptr);
-  float y[8];
+                     void* __restrict__ out, int64_t ostride, int mode) {
+  const int64_t opr = cols >> 3, total = rows * opr;
+  const int64_t o0 = (int64_t)blockIdx.x * (kT * kOct) + threadIdx.x;
+  uint32_t w[kOct], sb[kOct];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const uint32_t b = (w >> (8 * j)) & 0xFFu;
-    y[2 * j] = e2m1_value(b & 0xFu) * eff;
-    y[2 * j + 1] = e2m1_value(b >> 4) * eff;
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    w[k] = o < total ? packed[o] : 0u;
+    sb[k] = o < total ? (uint32_t)scale8[o >> 1] : 0u;
   }
-  store8<OUT>(out, row * ostride + c8 * 8, y);
+  const float gs = *gs_ptr;
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    const int64_t o = o0 + (int64_t)k * kT;
+    if (o >= total) continue;
+    const float eff = e4m3fn_bits_to_f32(sb[k]) * gs;
+    // v_cvt_scalef32_pk_f32_fp4: the two e2m1 values of one byte, exact in fp32
+    const f32x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[k], 1.0f, 0);
+    const f32x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[k], 1.0f, 1);
+    const f32x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[k], 1.0f, 2);
+    const f32x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[k], 1.0f, 3);
+    const float y[8] = {p0[0] * eff, p0[1] * eff, p1[0] * eff, p1[1] * eff,
+                        p2[0] * eff, p2[1] * eff, p3[0] * eff, p3[1] * eff};
+    store8<OUT>(out, octet_elem(o, opr, ostride, mode), y);
+  }
 }
 
 // One lane per 16-element block: any alignment.
@@ -674,6 +873,21 @@ inline bool valid_dt(int dt) { return dt == OA_F32 || dt == OA_BF16 || dt == OA_
 inline int64_t esize(int dt) { return dt == OA_F32 ? 4 : 2; }
 inline bool pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 inline unsigned blocks_for(int64_t work) { return (unsigned)((work + kT - 1) / kT); }
+inline unsigned blocks_oct(int64_t octets) {
+  return (unsigned)((octets + (int64_t)kT * kOct - 1) / ((int64_t)kT * kOct));
+}
+inline int addr_mode(int64_t rows, int64_t cols, int64_t stride) {
+  if (stride == cols || rows <= 1) return kFlat;
+  return rows * (cols / 8) < (int64_t(1) << 31) ? kDiv32 : kDiv64;
+}
+inline int div_mode(int64_t rows, int64_t cols) {  // when the row index itself is needed
+  return rows * (cols / 8) < (int64_t(1) << 31) ? kDiv32 : kDiv64;
+}
+inline int log2i(int64_t v) {
+  int s = 0;
+  while ((int64_t(1) << s) < v) ++s;
+  return s;
+}
 
 // fast path: rows of 8-element octets that all start on 16-byte boundaries
 inline bool rows_vec(const void* p, int dt, int64_t stride, int64_t cols) {
@@ -729,12 +943,12 @@ extern "C" int oa_dequant_int8(const void* q, const void* scales, int scale_dtyp
   if (!q || !scales) return OA_EINVAL;
   if (!aligned_to(scales, (uintptr_t)esize(scale_dtype))) return OA_EALIGN;
   const int vec = rows_vec(out, out_dtype, out_row_stride, cols) && aligned_to(q, 8);
-  const int64_t work = vec ? rows * (cols / 8) : rows * cols;
+  const unsigned blocks = vec ? blocks_oct(rows * (cols / 8)) : blocks_for(rows * cols);
   hipStream_t s = static_cast<hipStream_t>(stream);
   OA_DISPATCH_DT(out_dtype,
-                 hipLaunchKernelGGL(dequant_int8_kernel<DT>, dim3(blocks_for(work)), dim3(kT), 0,
+                 hipLaunchKernelGGL(dequant_int8_kernel<DT>, dim3(blocks), dim3(kT), 0,
                                     s, static_cast<const int8_t*>(q), scales, scale_dtype, rows,
-                                    cols, out, out_row_stride, vec));
+                                    cols, out, out_row_stride, vec, div_mode(rows, cols)));
   return launch_status();
 }
 
@@ -817,10 +1031,11 @@ extern "C" int oa_quant_nf4(const void* src, int src_dtype, int64_t src_row_stri
                     pow2(block / 8) && block <= 512 && aligned_to(packed, 4);
   if (fast) {
     OA_DISPATCH_DT(src_dtype,
-                   hipLaunchKernelGGL(quant_nf4_kernel<DT>, dim3(blocks_for(rows * (cols / 8))),
+                   hipLaunchKernelGGL(quant_nf4_kernel<DT>, dim3(blocks_oct(rows * (cols / 8))),
                                       dim3(kT), 0, s, src, src_row_stride, rows, cols,
-                                      (int)(block / 8), static_cast<uint32_t*>(packed),
-                                      static_cast<float*>(absmax)));
+                                      (int)(block / 8), log2i(block / 8),
+                                      static_cast<uint32_t*>(packed), static_cast<float*>(absmax),
+                                      addr_mode(rows, cols, src_row_stride)));
   } else {
     OA_DISPATCH_DT(src_dtype,
                    hipLaunchKernelGGL(quant_nf4_generic<DT>,
@@ -845,10 +1060,11 @@ extern "C" int oa_dequant_nf4(const void* packed, const void* absmax, int64_t ro
                     pow2(block / 8) && block <= 512 && aligned_to(packed, 4);
   if (fast) {
     OA_DISPATCH_DT(out_dtype,
-                   hipLaunchKernelGGL(dequant_nf4_kernel<DT>, dim3(blocks_for(rows * (cols / 8))),
+                   hipLaunchKernelGGL(dequant_nf4_kernel<DT>, dim3(blocks_oct(rows * (cols / 8))),
                                       dim3(kT), 0, s, static_cast<const uint32_t*>(packed),
                                       static_cast<const float*>(absmax), rows, cols,
-                                      (int)(block / 8), out, out_row_stride));
+                                      log2i(block / 8), out, out_row_stride,
+                                      addr_mode(rows, cols, out_row_stride)));
   } else {
     OA_DISPATCH_DT(out_dtype,
                    hipLaunchKernelGGL(dequant_nf4_generic<DT>,
@@ -882,17 +1098,19 @@ extern "C" int oa_quant_nvfp4(const void* src, int src_dtype, int64_t src_row_st
                                     partial));
   rc = launch_status();
   if (rc) return rc;
-  hipLaunchKernelGGL(nvfp4_global_scale_kernel, dim3(1), dim3(kT), 0, s, partial, (int)rblocks,
+  hipLaunchKernelGGL(nvfp4_global_scale_kernel, dim3(1), dim3(kScaleThreads), 0, s, partial,
+                     (int)rblocks,
                      static_cast<float*>(global_scale));
   rc = launch_status();
   if (rc || rows * cols == 0) return rc;
   if (vec && aligned_to(packed, 4) && aligned_to(block_scale, 4)) {
     OA_DISPATCH_DT(src_dtype,
-                   hipLaunchKernelGGL(quant_nvfp4_kernel<DT>, dim3(blocks_for(rows * (cols / 8))),
+                   hipLaunchKernelGGL(quant_nvfp4_kernel<DT>, dim3(blocks_oct(rows * (cols / 8))),
                                       dim3(kT), 0, s, src, src_row_stride, rows, cols,
                                       static_cast<uint32_t*>(packed),
                                       static_cast<uint8_t*>(block_scale),
-                                      static_cast<const float*>(global_scale)));
+                                      static_cast<const float*>(global_scale),
+                                      addr_mode(rows, cols, src_row_stride)));
   } else {
     OA_DISPATCH_DT(src_dtype,
                    hipLaunchKernelGGL(quant_nvfp4_generic<DT>,
@@ -918,11 +1136,11 @@ extern "C" int oa_dequant_nvfp4(const void* packed, const void* block_scale,
   if (rows_vec(out, out_dtype, out_row_stride, cols) && aligned_to(packed, 4)) {
     OA_DISPATCH_DT(out_dtype,
                    hipLaunchKernelGGL(dequant_nvfp4_kernel<DT>,
-                                      dim3(blocks_for(rows * (cols / 8))), dim3(kT), 0, s,
+                                      dim3(blocks_oct(rows * (cols / 8))), dim3(kT), 0, s,
                                       static_cast<const uint32_t*>(packed),
                                       static_cast<const uint8_t*>(block_scale),
                                       static_cast<const float*>(global_scale), rows, cols, out,
-                                      out_row_stride));
+                                      out_row_stride, addr_mode(rows, cols, out_row_stride)));
   } else {
     OA_DISPATCH_DT(out_dtype,
                    hipLaunchKernelGGL(dequant_nvfp4_generic<DT>,

@@ -24,7 +24,8 @@ namespace oa {
 namespace {
 
 constexpr int kThreads = 512;   // partial kernel
-constexpr int kFinalThreads = 256;
+constexpr int kFinalThreads = 1024;  // 4 partials per lane per trip: 16384 partials = 4 trips
+constexpr int kClipThreads = 256;
 constexpr int kUnroll = 4;      // 16-byte loads in flight per lane
 constexpr int kMaxBlocks = 16384;
 constexpr int64_t kTileGroups = (int64_t)kThreads * kUnroll;  // 8-element groups per tile
@@ -98,7 +99,15 @@ grad_norm_final_kernel(const float* __restrict__ partial, int blocks,
                        uint16_t* __restrict__ norm_out, float* __restrict__ sumsq_out) {
   __shared__ float lds[kFinalThreads / kWave];
   float s = 0.0f;
-  for (int b = threadIdx.x; b < blocks; b += kFinalThreads) s += partial[b];
+  for (int b = threadIdx.x; b < blocks; b += 4 * kFinalThreads) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = b + k * kFinalThreads;
+      v[k] = i < blocks ? partial[i] : 0.0f;
+    }
+    s += (v[0] + v[1]) + (v[2] + v[3]);
+  }
   s = block_sum<kFinalThreads>(s, lds);
   if (threadIdx.x == 0) {
     if (sumsq_out) *sumsq_out = s;
@@ -109,16 +118,16 @@ grad_norm_final_kernel(const float* __restrict__ partial, int blocks,
 // total = bf16(sqrt(sum norms^2)); coef = min(bf16(bf16(1/bf16(total+1e-6)) * max_norm), 1)
 // -- the bf16 0-dim tensor arithmetic of the reference's clip step, where
 // `python_float / tensor` is evaluated as `tensor.reciprocal() * python_float`.
-__global__ void __launch_bounds__(kFinalThreads)
+__global__ void __launch_bounds__(kClipThreads)
 clip_coef_kernel(const uint16_t* __restrict__ norms, int64_t count, float max_norm,
                  uint16_t* __restrict__ total_out, uint16_t* __restrict__ coef_out) {
-  __shared__ float lds[kFinalThreads / kWave];
+  __shared__ float lds[kClipThreads / kWave];
   float acc = 0.0f;
-  for (int64_t i = threadIdx.x; i < count; i += kFinalThreads) {
+  for (int64_t i = threadIdx.x; i < count; i += kClipThreads) {
     const float x = bf16_bits_to_f32(norms[i]);
     acc = fmaf(x, x, acc);
   }
-  const float s = block_sum<kFinalThreads>(acc, lds);
+  const float s = block_sum<kClipThreads>(acc, lds);
   if (threadIdx.x == 0) {
     const uint32_t total = f32_to_bf16_1(sqrtf(s));
     const uint32_t t1 = f32_to_bf16_1(bf16_bits_to_f32(total) + 1e-6f);
@@ -168,7 +177,7 @@ extern "C" int oa_clip_coef_bf16(const void* norms, int64_t count, float max_nor
   if (!aligned_to(norms, 2) || !aligned_to(coef_out, 2) ||
       (total_out && !aligned_to(total_out, 2)))
     return OA_EALIGN;
-  hipLaunchKernelGGL(clip_coef_kernel, dim3(1), dim3(kFinalThreads), 0,
+  hipLaunchKernelGGL(clip_coef_kernel, dim3(1), dim3(kClipThreads), 0,
                      static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(norms),
                      count, max_norm, static_cast<uint16_t*>(total_out),
                      static_cast<uint16_t*>(coef_out));

@@ -156,9 +156,10 @@ def test_strided_and_unaligned_sources(oracle):
 
 
 def test_nf4_thresholds_match_brute_force(oracle):
-    """The kernel's threshold tree must equal the 16-way fp32 distance search for
-    every input: all floats within 64 ulps of each decision point, the codebook
-    itself, and a dense sweep of [-1, 1]."""
+    """The kernel's threshold count (bucket table) must equal the 16-way fp32
+    distance search for every input: all floats within 64 ulps of each decision
+    point, within 8 ulps of every bucket edge k/128 - 1 (where the table index
+    changes), the codebook itself, and a dense sweep of [-1, 1]."""
     from offload_adam_amd.qweight import _codec_ops as ops
 
     lut = np.array([oracle.lib().oaref_nf4_lut(i) for i in range(16)], dtype=np.float32)
@@ -167,7 +168,15 @@ def test_nf4_thresholds_match_brute_force(oracle):
     for m in mids:
         b = int(m.view(np.uint32))
         pts.append(np.arange(b - 64, b + 65, dtype=np.uint32).view(np.float32))
+    for k in range(257):
+        e = np.float32(k / 128.0 - 1.0)
+        if e == 0:
+            pts.append(np.array([0.0, -0.0, 1e-45, -1e-45, 1e-38, -1e-38], dtype=np.float32))
+            continue
+        b = int(e.view(np.uint32))
+        pts.append(np.arange(b - 8, b + 9, dtype=np.uint32).view(np.float32))
     x = np.concatenate(pts)
+    x = x[np.abs(x) <= 1.0]  # each row's absmax must stay exactly 1
     pad = (-len(x)) % 64
     x = np.concatenate([x, np.zeros(pad, dtype=np.float32)])
     # one row per 64-block whose absmax is exactly 1, so normalised == input
@@ -181,6 +190,47 @@ def test_nf4_thresholds_match_brute_force(oracle):
     ops.quantize_nf4_into(t, 128, packed, absmax)
     rp, _ = oracle.quant_nf4(x, 128)
     assert np.array_equal(packed.cpu().numpy(), rp)
+
+
+def test_nvfp4_e2m1_boundaries_match_bit_level_definition(oracle):
+    """The vector kernel encodes with the GPU's FP4 conversion instruction; it must
+    agree with the bit-level e2m1 rounding (oracle) on every float within 64 ulps
+    of each grid point and rounding boundary, and on a dense sweep of [-6, 6].
+    Scales are forced to exactly 1: the tensor maximum is 448*6 (global scale 1)
+    and every 16-element block carries one 6.0 (block scale 1)."""
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    pts = [np.linspace(-6, 6, 120_001, dtype=np.float32)]
+    for v in (0.25, 0.5, 0.75, 1.0, 1.25, 1.5, 1.75, 2.0, 2.5, 3.0, 3.5, 4.0, 5.0, 6.0):
+        for sgn in (1.0, -1.0):
+            b = int(np.float32(sgn * v).view(np.uint32))
+            pts.append(np.arange(b - 64, b + 65, dtype=np.uint32).view(np.float32))
+    pts.append(np.array([0.0, -0.0, 1e-45, -1e-45, 1e-38, -1e-38, 1e-20], dtype=np.float32))
+    x = np.concatenate(pts)
+    x = x[np.abs(x) <= 6.0]
+    x = np.concatenate([x, np.zeros((-len(x)) % 15, dtype=np.float32)]).reshape(-1, 15)
+    blocks = np.concatenate([np.full((x.shape[0], 1), 6.0, dtype=np.float32), x], axis=1)
+    per_row = 8  # blocks per row -> 128 columns
+    pad = (-blocks.shape[0]) % per_row
+    blocks = np.concatenate([blocks, np.tile(blocks[:1], (pad, 1))])
+    mat = blocks.reshape(-1, per_row * 16)
+    top = np.zeros((1, per_row * 16), dtype=np.float32)
+    top[0, 0] = 448.0 * 6.0  # sets the tensor scale to exactly 1
+    mat = np.concatenate([top, mat])
+    t = torch.from_numpy(mat).cuda()
+    rows, cols = t.shape
+    packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    scales = torch.empty(rows, cols // 16, dtype=torch.float8_e4m3fn, device="cuda")
+    gs = torch.zeros((), dtype=torch.float32, device="cuda")
+    ops.quantize_nvfp4_into(t, packed, scales, gs)
+    assert float(gs) == 1.0
+    assert (scales[1:].view(torch.uint8) == 0x38).all()  # e4m3fn 1.0
+    rp, rs, rg = oracle.quant_nvfp4(mat)
+    assert np.array_equal(packed.cpu().numpy(), rp)
+    assert np.array_equal(scales.view(torch.uint8).cpu().numpy(), rs)
+    back = ops.dequantize_nvfp4(packed, scales, gs, cols, torch.float32)
+    assert np.array_equal(back.cpu().numpy().view(np.uint32),
+                          oracle.dequant_nvfp4(rp, rs, rg, "float32").view(np.uint32))
 
 
 def test_config3_weight(oracle):
