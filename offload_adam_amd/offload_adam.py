@@ -647,14 +647,34 @@ class OffloadAdam(Optimizer):
         copies, so they run under that forward pass instead of waiting for the
         first backward hook."""
         self._ready_for_optimizer_step = bool(value)
-        if (
-            self._ready_for_optimizer_step
-            and getattr(self, "_bw_order_known", False)
-            and self._step_in_backward
-            and self._bw_cursor < 0
-        ):
+        if not self._ready_for_optimizer_step or not hasattr(self, "_bw_order"):
+            return
+        if self._step_in_backward:
+            if self._bw_order_known and self._bw_cursor < 0:
+                with torch.no_grad():
+                    self._prefetch_ahead(-1)
+        else:
             with torch.no_grad():
-                self._prefetch_ahead(-1)
+                self._prestage_for_step()
+
+    def _prestage_for_step(self):
+        """Clip path: the states do not depend on the clip coefficient, so the
+        first ``prefetch_bytes`` of them (in the order ``step()`` walks the
+        parameters) cross the link under the last backward pass instead of
+        inside ``step()``."""
+        budget = self._PREFETCH_BYTES
+        per_elem = self._bytes_per_elem_in_flight - 2  # all states but the gradient
+        for group in self.param_groups:
+            for p in group["params"]:
+                if budget <= 0:
+                    return
+                if p in self._inplace_params:
+                    continue
+                dev = self.device_states[p]
+                missing = [k for k in self._non_grad_keys if dev.get(k) is None]
+                if missing:
+                    self._issue_h2d(p, missing)
+                budget -= p.numel() * per_elem
 
     def _pre_backward_hook(self, module, grad_output):
         # Idempotent across the several fires a backward can produce for one
