@@ -215,6 +215,16 @@ def run(args):
     out["link_peak"] = measure_link()
 
     model = build_model(cfg, dev)
+    if args.qat:
+        from offload_adam_amd import qweight
+
+        cls = {"int8": qweight.Int8QWeight, "int4": qweight.Int4QWeight,
+               "nf4": qweight.NF4QWeight, "nvfp4": qweight.NVFP4QWeight}[args.qat]
+        report = qweight.quantize_linears(model, cls, skip_patterns=("lm_head",))
+        out["qat"] = {"format": args.qat, "quantized_linears": len(report.quantized),
+                      "incompatible": len(report.incompatible)}
+        torch.cuda.empty_cache()
+        out["model_gpu_GiB"] = round(torch.cuda.memory_allocated() / 1024**3, 2)
     n_params = sum(p.numel() for p in model.parameters())
     out["params"] = n_params
     ids = [torch.randint(0, cfg["vocab"], (1, args.seq), device=dev,
@@ -292,12 +302,17 @@ def main():
     ap.add_argument("--one-transfer-stream", action="store_true")
     ap.add_argument("--prefetch-gib", type=float, default=None,
                     help="device staging budget of the H2D prefetch window")
+    ap.add_argument("--qat", default=None, choices=["int8", "int4", "nf4", "nvfp4"],
+                    help="quantise every decoder Linear weight (lm_head excluded) and train "
+                         "against fp32 masters: implies --mode fp32_master")
     ap.add_argument("--grads-on-device", action="store_true",
                     help="OffloadAdam(offload_grads=False): the gradient sum stays in HBM")
     ap.add_argument("--runtime-copy-engines", action="store_true",
                     help="leave the SDMA engine of each copy to the HIP runtime "
                          "(do not load the fixed-engine tools library)")
     args = ap.parse_args()
+    if args.qat:
+        args.mode = "fp32_master"
     if args.runtime_copy_engines:
         import os
 

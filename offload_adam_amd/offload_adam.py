@@ -21,6 +21,7 @@ What runs underneath is this package's HIP library: the fused AdamW kernels
 ``hipMemcpyAsync`` on two side streams fenced with events.
 """
 
+import bisect
 import time
 import warnings
 from ctypes import c_int, c_size_t, c_void_p
@@ -343,6 +344,8 @@ class OffloadAdam(Optimizer):
         self._bw_pos = {}
         self._bw_order_known = False
         self._bw_cursor = -1
+        self._bw_prefix = [0]
+        self._bw_issued_upto = 0
         self._bytes_per_elem_in_flight = sum(
             torch.empty(0, dtype=d).element_size() for d in self.offload_config.values()
         )
@@ -624,17 +627,32 @@ class OffloadAdam(Optimizer):
         backward kernels of earlier modules; without it a copy can only start
         when the compute stream reaches its own module (the fence against the
         compute stream is taken when a copy is issued) and the compute stream
-        then waits for it."""
+        then waits for it.
+
+        The window's far end only moves forward within a pass, so each call looks
+        at the parameters that newly entered it (a call with ``pos == -1`` starts
+        a pass and looks at the whole first window)."""
         order = self._bw_order
-        budget = self._PREFETCH_BYTES
-        j = pos + 1
-        while j < len(order) and (j - pos <= self._PREFETCH_MIN_PARAMS or budget > 0):
+        if len(self._bw_prefix) != len(order) + 1:
+            # bytes of device staging of order[:j], for the bisection below
+            self._bw_prefix = [0]
+            for q in order:
+                self._bw_prefix.append(
+                    self._bw_prefix[-1] + q.numel() * self._bytes_per_elem_in_flight
+                )
+        prefix = self._bw_prefix
+        first = pos + 1
+        # parameters j >= first are wanted while the bytes of order[first:j] stay
+        # below the budget, and in any case the next _PREFETCH_MIN_PARAMS
+        end = bisect.bisect_left(prefix, prefix[first] + self._PREFETCH_BYTES, lo=first)
+        end = min(len(order), max(end, first + self._PREFETCH_MIN_PARAMS))
+        start = first if pos < 0 else max(first, self._bw_issued_upto)
+        for j in range(start, end):
             q = order[j]
             keys = self._wanted_keys(q, states_too)
             if keys:
                 self._issue_h2d(q, keys)
-            budget -= q.numel() * self._bytes_per_elem_in_flight
-            j += 1
+        self._bw_issued_upto = max(end, 0 if pos < 0 else self._bw_issued_upto)
 
     @property
     def ready_for_optimizer_step(self):
