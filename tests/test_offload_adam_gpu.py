@@ -522,3 +522,63 @@ def test_prefetch_budget_does_not_change_results(fixed_seed, prefetch_bytes):
     model2, _ = run_offload_adam("stochastic_rounding", steps=4, ga=3,
                                  prefetch_bytes=prefetch_bytes, offload_grads=False)
     assert_same_params(ref_model, model2)
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(max_grad_norm=0.05), dict(offload_grads=False),
+                                dict(prefetch_bytes=0)])
+def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monkeypatch, kw):
+    """Log every H2D / kernel / D2H the optimizer issues and check, per parameter
+    and state key: a key is on the device (H2D issued, not yet written back) when
+    the kernel runs; it is written back after the kernel and before it is fetched
+    again; nothing is fetched twice without a write-back in between; each
+    offloaded parameter is stepped exactly once per optimizer step."""
+    from offload_adam_amd import offload_adam as oa_mod
+
+    log = []
+    real = {n: getattr(oa_mod.OffloadAdam, n) for n in ("_issue_h2d", "_issue_d2h", "_call_step_fn")}
+
+    def h2d(self, p, keys):
+        log.append(("h2d", p, tuple(keys)))
+        return real["_issue_h2d"](self, p, keys)
+
+    def d2h(self, p, keys):
+        log.append(("d2h", p, tuple(keys)))
+        return real["_issue_d2h"](self, p, keys)
+
+    def step(self, p, group, tensors, clip_coef=None):
+        log.append(("step", p, tuple(tensors)))
+        return real["_call_step_fn"](self, p, group, tensors, clip_coef)
+
+    monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_h2d", h2d)
+    monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_d2h", d2h)
+    monkeypatch.setattr(oa_mod.OffloadAdam, "_call_step_fn", step)
+    steps, ga = 3, 3
+    model, opt = run_offload_adam("fp31_master", steps=steps, ga=ga, **kw)
+    offloaded = set(opt._offload_params)
+    on_device = {}  # (param, key) -> True while a fetched copy is live
+    stepped = {p: 0 for p in offloaded}
+    for op, p, keys in log:
+        if p not in offloaded:
+            assert op == "step"  # GPU-resident parameters never cross the link
+            continue
+        if op == "h2d":
+            for k in keys:
+                assert not on_device.get((p, k)), f"{k} fetched twice without a write-back"
+                on_device[(p, k)] = True
+        elif op == "d2h":
+            for k in keys:
+                if k != "grad" or opt.offload_grads:
+                    on_device[(p, k)] = False
+        else:
+            stepped[p] += 1
+            for k in opt._non_grad_keys:
+                assert on_device.get((p, k)), f"kernel ran without {k} on the device"
+            if opt.offload_grads and ga > 1:
+                assert on_device.get((p, "grad")), "kernel ran without the accumulated gradient"
+    assert set(stepped.values()) == {steps}
+    # at the end of a step nothing but staged states of the next step is live, and
+    # every state written by a kernel went back to the host
+    last_step_index = max(i for i, e in enumerate(log) if e[0] == "step" and e[1] in offloaded)
+    written_back = {(p, k) for op, p, keys in log[last_step_index:] if op == "d2h" for k in keys}
+    p_last = log[last_step_index][1]
+    assert {(p_last, k) for k in opt._non_grad_keys} <= written_back
