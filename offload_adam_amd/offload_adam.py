@@ -29,7 +29,7 @@ from ctypes import c_int, c_size_t, c_void_p
 import torch
 from torch.optim.optimizer import Optimizer
 
-from . import _copy_engines, _lib, grad_clip
+from . import _copy_engines, _lib, _trace, grad_clip
 from ._pretrained import stream_master_from_pretrained
 from .adam import _LOSSY_MASTER_HINT, MODE_TABLE
 from .kernels import adam_step_multi
@@ -720,6 +720,13 @@ class OffloadAdam(Optimizer):
             self._bw_order.append(p)
         else:
             self._bw_order_known = True  # a second pass has begun
+        if _trace.ENABLED:
+            with _trace.range(f"oa.hook #{pos} {tuple(p.shape)}"):
+                self._grad_hook_body(p, pos)
+        else:
+            self._grad_hook_body(p, pos)
+
+    def _grad_hook_body(self, p, pos):
         if self._bw_order_known:
             self._bw_cursor = -1 if pos == len(self._bw_order) - 1 else pos
             self._prefetch_ahead(pos)
@@ -797,7 +804,8 @@ class OffloadAdam(Optimizer):
                 if missing:
                     self._issue_h2d(q, missing)
                 ahead += 1
-            self._step_offload(p, group, clip_coef)
+            with _trace.range(f"oa.step #{done} {tuple(p.shape)}"):
+                self._step_offload(p, group, clip_coef)
             state["host_grad_valid"] = False
             done += 1
 

@@ -103,3 +103,18 @@ def test_copies_run_on_the_fixed_engines_and_move_the_right_bytes():
     assert st1["h2d_copies"] - st0["h2d_copies"] >= 4
     assert st1["d2h_copies"] - st0["d2h_copies"] >= 4
     assert st1["rejected"] == 0 and st1["active"]
+
+
+def test_roctx_ranges_are_off_by_default_and_load_on_request():
+    from offload_adam_amd import _trace
+
+    if not _trace.ENABLED:
+        with _trace.range("nothing"):  # a null context
+            pass
+    code = ("from offload_adam_amd import _trace\n"
+            "with _trace.range('outer'):\n"
+            "    with _trace.range('inner'):\n"
+            "        pass\n"
+            "print(_trace.ENABLED)")
+    assert _run(code, OFFLOAD_ADAM_ROCTX="1") == "True"
+    assert _run(code) == "False"
