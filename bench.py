@@ -108,9 +108,10 @@ def make_tensors(mode, shapes, device, seed=0):
     return out
 
 
-def cpu_baseline(mode, target_elems=32 * 1024 * 1024, iters=3):
+def cpu_baseline(mode, target_elems=256 * 1024 * 1024, iters=5):
     """The same update math in PyTorch eager on this host's cores, on a bounded
-    sample of the workload (one flat tensor of ``target_elems`` elements)."""
+    sample of the workload: one flat tensor of ``target_elems`` elements (a
+    quarter of config 1), ``iters`` timed passes of about 2 s each."""
     import torch
 
     from oracle import folded_betas, torch_eager
