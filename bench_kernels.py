@@ -4,15 +4,16 @@ AdamW launch that ``bench.py`` measures: gradient L2 norm, clip coefficient,
 the fused AdamW kernel with the clip coefficient folded in (fp31_master), and
 the eight weight codecs.  One JSON line per kernel.
 
-    python bench_kernels.py [--reps 20] [--only norm,clip,adam,codecs]
+    python bench_kernels.py [--reps 20] [--only norm_large,norm_small,clip,adam,codecs]
 
 Shapes: the offloaded parameters of a Llama-3-8B-shaped decoder for the norm
 and AdamW kernels, one 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
 x10 for the codecs.  Every launch works on buffers that were not touched by the
 previous launches of the same kernel (the inputs rotate through more distinct
 buffers than the 256 MiB memory-side cache holds), so the figures are HBM
-figures.  ``achieved`` = algorithmic bytes of one launch / its duration between
-two HIP events on the launch stream; ``frac`` is against 8 TB/s.
+figures.  ``achieved`` = algorithmic bytes of one launch / (time between two HIP
+events around ``--reps`` back-to-back launches on the launch stream / reps);
+``frac`` is against 8 TB/s.
 """
 
 import argparse
@@ -28,19 +29,23 @@ ROWS, COLS = 4096, 14336
 
 
 def timed(fn, reps, torch):
-    """fn(i) launches once on rotation slot i; returns average microseconds."""
+    """fn(i) launches once on rotation slot i; returns microseconds per launch.
+
+    The launches are issued back to back between ONE pair of events: while the
+    host keeps ahead of the GPU (true for every kernel here longer than the
+    ~15 us a Python launch costs) the interval is GPU time, launch gaps included;
+    for shorter kernels it is the host's launch rate, and says so in the
+    profiler summary under profiles/."""
     for i in range(3):
         fn(i)
     torch.cuda.synchronize()
-    evs = []
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
     for i in range(reps):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
         fn(i)
-        b.record()
-        evs.append((a, b))
+    b.record()
     torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in evs) / reps * 1e3
+    return a.elapsed_time(b) / reps * 1e3
 
 
 def line(kernel, workload, alg_bytes, us, **extra):
@@ -59,22 +64,31 @@ def outlier_weight(torch, seed, dtype):
     return torch.where(mask, w * 10, w).to(dtype)
 
 
-def bench_norm_and_clip(args, torch):
+def bench_norm_and_clip(args, torch, todo):
     from offload_adam_amd import grad_clip
 
+    if "norm_large" in todo:
+        bench_norm_large(args, torch, grad_clip)
+    if "norm_small" in todo:
+        norms = torch.zeros(1, dtype=torch.bfloat16, device="cuda")
+        small = torch.randn(4096 * 1024, device="cuda", dtype=torch.bfloat16)
+        us = timed(lambda i: grad_clip.grad_norm_(small, norms[0]), args.reps, torch)
+        line("grad_norm_partial_kernel + grad_norm_final_kernel",
+             "bf16 gradient 1024x4096 (cache resident)", 2 * small.numel(), us)
+    if "clip" in todo:
+        per_param = torch.rand(291, device="cuda").to(torch.bfloat16)
+        coef = torch.ones((), dtype=torch.bfloat16, device="cuda")
+        us = timed(lambda i: grad_clip.clip_coef_(per_param, 1.0, coef), args.reps, torch)
+        line("clip_coef_kernel", "291 per-parameter norms", 2 * 291, us, bound="latency")
+
+
+def bench_norm_large(args, torch, grad_clip):
     n_big = COLS * 4096
     slots = 8  # 8 x 117 MB = 0.94 GB rotation
     grads = [torch.randn(n_big, device="cuda", dtype=torch.bfloat16) * 5e-3 for _ in range(slots)]
     norms = torch.zeros(slots, dtype=torch.bfloat16, device="cuda")
     us = timed(lambda i: grad_clip.grad_norm_(grads[i % slots], norms[i % slots]), args.reps, torch)
     line("grad_norm_partial_kernel + grad_norm_final_kernel", "bf16 gradient 14336x4096", 2 * n_big, us)
-    small = torch.randn(4096 * 1024, device="cuda", dtype=torch.bfloat16)
-    us = timed(lambda i: grad_clip.grad_norm_(small, norms[0]), args.reps, torch)
-    line("grad_norm_partial_kernel + grad_norm_final_kernel", "bf16 gradient 1024x4096 (cache resident)", 2 * small.numel(), us)
-    per_param = torch.rand(291, device="cuda").to(torch.bfloat16)
-    coef = torch.ones((), dtype=torch.bfloat16, device="cuda")
-    us = timed(lambda i: grad_clip.clip_coef_(per_param, 1.0, coef), args.reps, torch)
-    line("clip_coef_kernel", "291 per-parameter norms", 2 * 291, us, bound="latency")
 
 
 def bench_adam_clip(args, torch):
@@ -161,8 +175,9 @@ def bench_codecs(args, torch):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--reps", type=int, default=20)
-    ap.add_argument("--only", default="norm,adam,codecs")
+    ap.add_argument("--reps", type=int, default=40)
+    ap.add_argument("--only", default="norm_large,norm_small,clip,adam,codecs",
+                    help="comma-separated subset of: norm_large, norm_small, clip, adam, codecs")
     args = ap.parse_args()
 
     import torch
@@ -175,8 +190,8 @@ def main():
     _lib.load()
     torch.cuda.set_device(0)
     todo = set(args.only.split(","))
-    if "norm" in todo:
-        bench_norm_and_clip(args, torch)
+    if todo & {"norm_large", "norm_small", "clip"}:
+        bench_norm_and_clip(args, torch, todo)
     if "adam" in todo:
         bench_adam_clip(args, torch)
     if "codecs" in todo:

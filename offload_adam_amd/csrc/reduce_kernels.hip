@@ -23,10 +23,16 @@
 namespace oa {
 namespace {
 
-constexpr int kThreads = 512;   // partial kernel
+#ifndef OA_NORM_THREADS
+#define OA_NORM_THREADS 512
+#endif
+#ifndef OA_NORM_UNROLL
+#define OA_NORM_UNROLL 4
+#endif
+constexpr int kThreads = OA_NORM_THREADS;   // partial kernel
 constexpr int kFinalThreads = 1024;  // 4 partials per lane per trip: 16384 partials = 4 trips
 constexpr int kClipThreads = 256;
-constexpr int kUnroll = 4;      // 16-byte loads in flight per lane
+constexpr int kUnroll = OA_NORM_UNROLL;  // 16-byte loads in flight per lane
 constexpr int kMaxBlocks = 16384;
 constexpr int64_t kTileGroups = (int64_t)kThreads * kUnroll;  // 8-element groups per tile
 
