@@ -199,6 +199,75 @@ def link_bytes_per_step(opt, grad_accum):
     return h2d, d2h
 
 
+class CopyTimeline:
+    """Times every copy the optimizer issues with a pair of events on the copy's own
+    stream (the profiler cannot be used for this: under rocprofv3 the copy-engine
+    tools library is not loaded).  ``summary()`` covers the copies of the last
+    ``steps`` optimizer steps."""
+
+    def __init__(self, torch, oa_mod):
+        self.torch, self.oa_mod, self.log = torch, oa_mod, []
+        self._orig = oa_mod._copy_async
+        oa_mod._copy_async = self._timed_copy
+
+    def _timed_copy(self, dst, src, kind, stream):
+        e0 = self.torch.cuda.Event(enable_timing=True)
+        e1 = self.torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        self._orig(dst, src, kind, stream)
+        e1.record(stream)
+        self.log.append((kind, src.numel() * src.element_size(), e0, e1))
+
+    def mark(self):
+        self.first = len(self.log)
+
+    def close(self):
+        self.oa_mod._copy_async = self._orig
+
+    @staticmethod
+    def _union(iv):
+        out = []
+        for s, e in sorted(iv):
+            if out and s <= out[-1][1]:
+                out[-1][1] = max(out[-1][1], e)
+            else:
+                out.append([s, e])
+        return out
+
+    def summary(self, steps):
+        rows = self.log[self.first:]
+        if not rows:
+            return None
+        base = rows[0][2]
+        iv = {0: [], 1: []}
+        big = {0: [], 1: []}
+        for kind, nbytes, e0, e1 in rows:
+            s, e = base.elapsed_time(e0), base.elapsed_time(e1)
+            iv[kind].append((s, e))
+            if nbytes >= 100e6 and e > s:
+                big[kind].append(nbytes / (e - s) / 1e6)
+        uh, ud = self._union(iv[0]), self._union(iv[1])
+        both, i, j = 0.0, 0, 0
+        while i < len(uh) and j < len(ud):
+            lo, hi = max(uh[i][0], ud[j][0]), min(uh[i][1], ud[j][1])
+            both += max(0.0, hi - lo)
+            if uh[i][1] < ud[j][1]:
+                i += 1
+            else:
+                j += 1
+        med = lambda v: round(sorted(v)[len(v) // 2], 1) if v else None  # noqa: E731
+        return {
+            "copies_per_step": len(rows) // steps,
+            "h2d_busy_s_per_step": round(sum(e - s for s, e in uh) / 1e3 / steps, 3),
+            "d2h_busy_s_per_step": round(sum(e - s for s, e in ud) / 1e3 / steps, 3),
+            "both_busy_s_per_step": round(both / 1e3 / steps, 3),
+            "h2d_GBps_median_large_copy": med(big[0]),
+            "d2h_GBps_median_large_copy": med(big[1]),
+            "h2d_GBps_min_large_copy": round(min(big[0]), 1) if big[0] else None,
+            "d2h_GBps_min_large_copy": round(min(big[1]), 1) if big[1] else None,
+        }
+
+
 def run(args):
     import torch
 
@@ -266,9 +335,19 @@ def run(args):
     out["inplace_params"] = len(opt._inplace_params)
     out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
 
+    timeline = None
+    if args.copy_timeline:
+        from offload_adam_amd import offload_adam as oa_mod
+
+        timeline = CopyTimeline(torch, oa_mod)
     torch.cuda.reset_peak_memory_stats()
     loop(opt, args.warmup)
+    if timeline:
+        timeline.mark()
     step_s = loop(opt, args.steps)
+    if timeline:
+        timeline.close()
+        out["copy_timeline"] = timeline.summary(args.steps)
     out["step_s"] = round(step_s, 4)
     out["tokens_per_s"] = round(args.grad_accum * args.seq / step_s, 1)
     out["exposed_optimizer_s"] = round(step_s - out["fwd_bwd_only_s"], 4)
@@ -307,6 +386,9 @@ def main():
                          "against fp32 masters: implies --mode fp32_master")
     ap.add_argument("--grads-on-device", action="store_true",
                     help="OffloadAdam(offload_grads=False): the gradient sum stays in HBM")
+    ap.add_argument("--copy-timeline", action="store_true",
+                    help="time every optimizer copy with events on its stream and report link "
+                         "occupancy per direction (adds two event records per copy)")
     ap.add_argument("--runtime-copy-engines", action="store_true",
                     help="leave the SDMA engine of each copy to the HIP runtime "
                          "(do not load the fixed-engine tools library)")
