@@ -157,6 +157,30 @@ def cpu_baseline(mode, target_elems=256 * 1024 * 1024, iters=5):
     }
 
 
+def offloaded_step_8b(timeout_s=420):
+    """The second half of the metric: step time of a synthetic Llama-3-8B-shaped
+    training step through OffloadAdam (BASELINE config 4), measured by
+    bench_e2e.py in a child process.  PCIe-inclusive; never part of ``value``."""
+    import subprocess
+
+    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", "2",
+           "--warmup", "1"]
+    try:
+        res = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout_s, cwd=str(ROOT))
+        if res.returncode != 0:
+            return {"error": f"bench_e2e.py exited with {res.returncode}",
+                    "stderr_tail": res.stderr[-300:]}
+        full = json.loads(res.stdout.strip().splitlines()[-1])
+    except Exception as exc:  # a failed side measurement must not lose the main line
+        return {"error": repr(exc)[:300]}
+    keep = ("model", "mode", "seq", "grad_accum", "offload_grads", "params", "step_s",
+            "tokens_per_s", "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step",
+            "d2h_GB_per_step", "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak",
+            "link_floor_s", "pinned_GiB", "peak_gpu_GiB", "optimizer_init_s", "copy_engines",
+            "transfer_streams")
+    return {k: full[k] for k in keep if k in full}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,6 +195,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run three 1 GiB device copies first (reference for counter runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip the 8B offloaded training step (bench_e2e.py, run as a child "
+                         "process after the timed region; about a minute)")
     ap.add_argument("--no-events", action="store_true",
                     help="skip per-launch HIP events (used for profiler runs)")
     args = ap.parse_args()
@@ -314,6 +341,10 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(mode)
+    if not args.no_e2e and args.workload == "c1_sr_llama1b":
+        del tensors, p_list, st_list
+        torch.cuda.empty_cache()
+        out["offloaded_step_8b"] = offloaded_step_8b()
     print(json.dumps(out))
 
 
