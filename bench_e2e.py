@@ -333,6 +333,7 @@ def run(args):
     out["optimizer_init_s"] = round(time.perf_counter() - t0, 2)
     out["offloaded_params"] = len(opt._offload_params)
     out["inplace_params"] = len(opt._inplace_params)
+    out["prefetch_GiB"] = round(opt._PREFETCH_BYTES / 1024**3, 2)
     out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
 
     timeline = None

@@ -206,7 +206,9 @@ class OffloadAdam(Optimizer):
             shared by several modules, e.g. tied embeddings).
         verbose (int): non-zero prints the pinned / in-place byte totals.
         prefetch_bytes (int, keyword-only): device staging the hook path may fill
-            ahead of the gradient hooks (default 8 GiB).  The copies of a
+            ahead of the gradient hooks.  Default: a tenth of the HBM that is free
+            when the optimizer is built (at least 2 GiB) - 27 GiB next to an 8B
+            model on a 288 GB MI355X, which holds most of that model's states.  The copies of a
             parameter's states start this far ahead in backward order; once a
             step completes, the first ``prefetch_bytes`` of the next step's
             states are staged straight away and wait in HBM through the
@@ -233,7 +235,7 @@ class OffloadAdam(Optimizer):
     _DEFAULT_INPLACE_PARAM_THRESHOLD = 1024 * 1024
     _CLIP_PREFETCH_DEPTH = 2  # parameters whose H2D runs ahead of the step loop
     _PREFETCH_MIN_PARAMS = 2  # hook path: H2D window ahead of the gradient hooks ...
-    _PREFETCH_BYTES = 8 << 30  # ... in parameters and in bytes of device staging
+    _PREFETCH_BYTES = 8 << 30  # ... and in bytes of device staging (re-derived per instance)
 
     def __init__(
         self,
@@ -265,6 +267,7 @@ class OffloadAdam(Optimizer):
         self.offload_state_keys = list(self.offload_config)
         self._non_grad_keys = [k for k in self.offload_state_keys if k != "grad"]
         self.offload_grads = bool(offload_grads)
+        self._prefetch_bytes_arg = prefetch_bytes
         if prefetch_bytes is not None:
             self._PREFETCH_BYTES = int(prefetch_bytes)
         # what lives in pinned host memory between steps
@@ -315,6 +318,13 @@ class OffloadAdam(Optimizer):
             if p.numel() < inplace_param_threshold and p not in self._quant_params
         }
         self._offload_params = [p for p in params if p not in self._inplace_params]
+
+        if self._prefetch_bytes_arg is None and self._offload_params:
+            # a tenth of what is free now (the model is already on the GPU), at least 2 GiB
+            dev0 = self._offload_params[0].device
+            if dev0.type == "cuda":
+                free, _ = torch.cuda.mem_get_info(dev0)
+                self._PREFETCH_BYTES = max(2 << 30, free // 10)
 
         self.device_states = {}
         self.h2d_events = {}
