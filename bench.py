@@ -163,7 +163,7 @@ def offloaded_step_8b(timeout_s=420):
     bench_e2e.py in a child process.  PCIe-inclusive; never part of ``value``."""
     import subprocess
 
-    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", "2",
+    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", "6",
            "--warmup", "1"]
     try:
         res = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout_s, cwd=str(ROOT))
@@ -173,7 +173,8 @@ def offloaded_step_8b(timeout_s=420):
         full = json.loads(res.stdout.strip().splitlines()[-1])
     except Exception as exc:  # a failed side measurement must not lose the main line
         return {"error": repr(exc)[:300]}
-    keep = ("model", "mode", "seq", "grad_accum", "offload_grads", "params", "step_s",
+    full["steps"], full["warmup"] = 6, 1
+    keep = ("model", "mode", "steps", "warmup", "seq", "grad_accum", "offload_grads", "params", "step_s",
             "tokens_per_s", "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step",
             "d2h_GB_per_step", "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak",
             "link_floor_s", "pinned_GiB", "prefetch_GiB", "peak_gpu_GiB", "optimizer_init_s", "copy_engines",
