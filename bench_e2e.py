@@ -321,6 +321,9 @@ def run(args):
     loop(None, 1)
     out["fwd_bwd_only_s"] = round(loop(None, args.steps), 4)
 
+    if args.optimizer == "adam":
+        return run_resident_adam(args, out, model, loop, torch)
+
     # 2) the offloaded optimizer
     t0 = time.perf_counter()
     with warnings.catch_warnings():
@@ -368,6 +371,31 @@ def run(args):
     return out
 
 
+def run_resident_adam(args, out, model, loop, torch):
+    """Same loop with ``Adam``: gradients accumulate in ``p.grad``, states stay in HBM."""
+    from offload_adam_amd import Adam
+
+    class Stepper:
+        def __init__(self, opt):
+            self.opt, self.ready_for_optimizer_step = opt, False
+
+        def step(self):
+            self.opt.step()
+
+        def zero_grad(self):
+            self.opt.zero_grad(set_to_none=True)
+
+    opt = Stepper(Adam(model.parameters(), lr=1e-5, mode=args.mode, decoupled_weight_decay=True))
+    torch.cuda.reset_peak_memory_stats()
+    loop(opt, args.warmup)
+    step_s = loop(opt, args.steps)
+    out.update(optimizer="adam", step_s=round(step_s, 4),
+               tokens_per_s=round(args.grad_accum * args.seq / step_s, 1),
+               exposed_optimizer_s=round(step_s - out["fwd_bwd_only_s"], 4),
+               peak_gpu_GiB=round(torch.cuda.max_memory_allocated() / 1024**3, 2))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--model", default="llama8b", choices=sorted(MODELS))
@@ -382,6 +410,9 @@ def main():
     ap.add_argument("--one-transfer-stream", action="store_true")
     ap.add_argument("--prefetch-gib", type=float, default=None,
                     help="device staging budget of the H2D prefetch window")
+    ap.add_argument("--optimizer", default="offload", choices=["offload", "adam"],
+                    help="'adam': the GPU-resident Adam of this package (states in HBM, "
+                         "multi-tensor launches in step()) instead of OffloadAdam")
     ap.add_argument("--qat", default=None, choices=["int8", "int4", "nf4", "nvfp4"],
                     help="quantise every decoder Linear weight (lm_head excluded) and train "
                          "against fp32 masters: implies --mode fp32_master")
