@@ -6,7 +6,6 @@ evaluation (and of torch.norm itself); everything downstream of the total
 (the coefficient, the clipped gradient inside the Adam kernel) is bit-exact.
 """
 
-import numpy as np
 import pytest
 import torch
 

@@ -12,7 +12,6 @@ import gc
 import random
 import warnings
 
-import numpy as np
 import pytest
 import torch
 import torch.nn as nn
