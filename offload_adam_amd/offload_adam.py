@@ -689,7 +689,14 @@ class OffloadAdam(Optimizer):
         """Clip path: the states do not depend on the clip coefficient, so the
         first ``prefetch_bytes`` of them (in the order ``step()`` walks the
         parameters) cross the link under the last backward pass instead of
-        inside ``step()``."""
+        inside ``step()``.  Not when this pass has to fetch accumulated gradients
+        from the host: the host->device direction is then busy for the whole pass
+        and staged states would only queue ahead of the gradients backward waits
+        for (measured: 2.86 s instead of 2.71 s per 8B step)."""
+        if self.offload_grads and any(
+            self.state[p]["host_grad_valid"] for p in self._offload_params
+        ):
+            return
         budget = self._PREFETCH_BYTES
         per_elem = self._bytes_per_elem_in_flight - 2  # all states but the gradient
         for group in self.param_groups:
