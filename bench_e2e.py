@@ -407,7 +407,6 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--d2h-workgroups", type=int, default=None,
                     help="workgroups of the write-back copy kernel (default: the optimizer's)")
-    ap.add_argument("--one-transfer-stream", action="store_true")
     ap.add_argument("--prefetch-gib", type=float, default=None,
                     help="device staging budget of the H2D prefetch window")
     ap.add_argument("--optimizer", default="offload", choices=["offload", "adam"],
@@ -431,10 +430,6 @@ def main():
         import os
 
         os.environ["OFFLOAD_ADAM_COPY_ENGINES"] = "off"  # before the package is imported
-    if args.one_transfer_stream:
-        from offload_adam_amd import offload_adam as _oa_mod
-
-        _oa_mod._ONE_TRANSFER_STREAM = args.one_transfer_stream
     if args.d2h_workgroups:
         from offload_adam_amd import offload_adam as _oa_mod
 

@@ -63,7 +63,6 @@ def _copy_async(dst, src, kind, stream):
     _lib.check(code, "oa_memcpy_async")
 
 
-_ONE_TRANSFER_STREAM = False  # queue both directions on one side stream
 _copy_engine_warned = False
 _D2H_BY_KERNEL = False  # write-back engine: DMA (default) or the library's copy kernel
 _D2H_WORKGROUPS = 8  # 1024-lane workgroups: enough requests in flight to fill the host link
@@ -332,7 +331,7 @@ class OffloadAdam(Optimizer):
         self.transfer_stream_report = None
         if self._offload_params:
             self._check_copy_engines()
-        if self._offload_params and _PROBE_TRANSFER_STREAMS and not _ONE_TRANSFER_STREAM:
+        if self._offload_params and _PROBE_TRANSFER_STREAMS:
             self.h2d_stream, self.d2h_stream, self.transfer_stream_report = pick_transfer_streams(
                 self._offload_params[0].device
             )
@@ -340,7 +339,7 @@ class OffloadAdam(Optimizer):
                 print(f"Transfer streams: {self.transfer_stream_report}")
         else:
             self.h2d_stream = torch.cuda.Stream()
-            self.d2h_stream = self.h2d_stream if _ONE_TRANSFER_STREAM else torch.cuda.Stream()
+            self.d2h_stream = torch.cuda.Stream()
         self._param2group = {p: g for g in self.param_groups for p in g["params"]}
         # first module in forward order that owns each offloaded param ('lazy' policy)
         self._prefetch_module = {}
