@@ -1,0 +1,151 @@
+"""The data in tests/golden/known_answers.json against the CPU oracle, and - for
+the codec entries - against the HIP kernels through the C ABI (``gpu`` tests)."""
+
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "known_answers.json").read_text())
+
+
+def h(x):
+    return int(x, 16)
+
+
+# ------------------------------------------------------------------ oracle
+
+
+def test_oracle_philox_and_triton_layout(oracle):
+    for kat in GOLDEN["philox4x32_10"]:
+        got = oracle.philox(tuple(map(h, kat["counter"])), tuple(map(h, kat["key"])))
+        assert got == tuple(map(h, kat["output"]))
+    seed = h(GOLDEN["triton_randint"]["seed"])
+    for offset, word in GOLDEN["triton_randint"]["words"].items():
+        assert oracle.lib().oaref_triton_randint(seed, int(offset)) == h(word)
+        assert oracle.lib().oaref_rand16(seed, int(offset), 0) == h(word) & 0xFFFF
+
+
+def test_oracle_folded_betas(oracle):
+    g = GOLDEN["folded_betas"]
+    b1, b2 = oracle.folded_betas(g["beta1"], g["beta2"], g["step"])
+    assert b1 == pytest.approx(g["beta1_hat"], rel=1e-15)
+    assert b2 == pytest.approx(g["beta2_hat"], rel=1e-15)
+
+
+def test_oracle_codec_anchors(oracle):
+    a = GOLDEN["int8_anchor"]
+    q, s = oracle.quant_int8(np.array([a["row"]], dtype=np.float32))
+    assert q[0].tolist() == a["codes"]
+    assert s[0] == np.float32(np.float32(a["scale_numerator"]) / np.float32(a["scale_denominator"]))
+    a = GOLDEN["int4_anchor"]
+    qw, s = oracle.quant_int4(np.array([a["row"]], dtype=np.float32), group=a["group"])
+    assert int(qw[0, 0]) & 0xFFFFFFFF == h(a["packed_word"]) and s[0, 0] == a["scale"]
+    lut = [oracle.lib().oaref_nf4_lut(i) for i in range(16)]
+    assert lut == [float(np.float32(v)) for v in GOLDEN["nf4_lut"]]
+    assert lut == sorted(lut) and lut[0] == -1.0 and lut[7] == 0.0 and lut[15] == 1.0
+
+
+def fp4_cases():
+    mags = np.array([c["magnitude"] for c in GOLDEN["fp4_rne_boundaries"]], dtype=np.float32)
+    want = np.array([c["expected_magnitude"] for c in GOLDEN["fp4_rne_boundaries"]],
+                    dtype=np.float32)
+    return mags, want
+
+
+def test_oracle_fp4_boundaries_and_signed_zero(oracle):
+    lut = np.array(GOLDEN["fp4_e2m1_lut"], dtype=np.float32)
+    mags, want = fp4_cases()
+    assert len(mags) == 30
+    for sign in (1.0, -1.0):
+        codes = oracle.fp4_code_array((mags * np.float32(sign)).astype(np.float32))
+        assert np.array_equal(np.abs(lut[codes]), want)
+        assert np.array_equal(codes >> 3, np.signbit(mags * np.float32(sign)).astype(codes.dtype))
+    z = oracle.fp4_code_array(np.array([0.0, -0.0], dtype=np.float32))
+    assert z.tolist() == [GOLDEN["fp4_signed_zero"]["+0.0"], GOLDEN["fp4_signed_zero"]["-0.0"]]
+
+
+# --------------------------------------------------------------- HIP kernels
+
+
+@pytest.mark.gpu
+def test_hip_int8_and_int4_anchors():
+    from offload_adam_amd.qweight import Int4QWeight, Int8QWeight
+
+    a = GOLDEN["int8_anchor"]
+    q = Int8QWeight.from_float(torch.tensor([a["row"]], device="cuda"), scale_dtype=torch.float32)
+    assert q.weight.cpu()[0].tolist() == a["codes"]
+    assert float(q.scales[0]) == float(np.float32(a["scale_numerator"]) /
+                                       np.float32(a["scale_denominator"]))
+    a = GOLDEN["int4_anchor"]
+    q = Int4QWeight.from_float(torch.tensor([a["row"]], dtype=torch.float32, device="cuda"),
+                               group_size=a["group"], scale_dtype=torch.float32)
+    assert int(q.qweight[0, 0]) & 0xFFFFFFFF == h(a["packed_word"])
+    assert float(q.scales[0, 0]) == a["scale"]
+
+
+@pytest.mark.gpu
+def test_hip_nf4_anchor_and_lut():
+    from offload_adam_amd.qweight import NF4QWeight
+
+    lut = torch.tensor(GOLDEN["nf4_lut"], dtype=torch.float32)
+    row = torch.zeros(1, 64)
+    row[0, :8] = lut[:8]      # codes 0..7 once the block's absmax is 1
+    row[0, 63] = 1.0
+    q = NF4QWeight.from_float(row.cuda(), blocksize=64)
+    assert q.weight_packed.cpu()[0, :4].tolist() == [h(b) for b in GOLDEN["nf4_anchor"]["packed_bytes"]]
+    back = q.dequantize(torch.float32).cpu()
+    assert torch.equal(back[0, :8], lut[:8]) and float(back[0, 63]) == 1.0
+    # every code decodes to its table entry
+    full = torch.cat([lut, torch.zeros(48)]).reshape(1, 64).cuda()
+    assert torch.equal(NF4QWeight.from_float(full, blocksize=64).dequantize(torch.float32).cpu()[0, :16], lut)
+
+
+@pytest.mark.gpu
+def test_hip_fp4_anchor_boundaries_and_signed_zero():
+    """Scales forced to exactly 1 (tensor maximum 448*6, one 6.0 opening every
+    16-element block), so the stored codes are the e2m1 codes of the inputs."""
+    from offload_adam_amd.qweight import NVFP4QWeight
+
+    lut = np.array(GOLDEN["fp4_e2m1_lut"], dtype=np.float32)
+    mags, want = fp4_cases()
+    keep = mags <= 6.0  # the 1e6 case owns the tensor scale: checked separately below
+    mags, want = mags[keep], want[keep]
+    assert len(mags) == 29
+
+    def block(vals):
+        return np.concatenate([[6.0], vals, np.zeros(15 - len(vals))]).astype(np.float32)
+
+    top = np.zeros(16, dtype=np.float32)
+    top[0] = 448.0 * 6.0
+    rows = [top,
+            block(mags[:15]), block(mags[15:]),          # rows 1, 2: positive
+            block(-mags[:15]), block(-mags[15:]),        # rows 3, 4: negative
+            block(np.concatenate([lut[:8], [0.0, -0.0]]).astype(np.float32))]  # row 5
+    q = NVFP4QWeight.from_float(torch.from_numpy(np.stack(rows)).cuda())
+    assert float(q.global_scale) == 1.0
+    assert (q.block_scale_fp8[1:].view(torch.uint8) == 0x38).all()  # e4m3fn 1.0
+    packed = q.weight_packed.cpu().numpy()
+    codes = np.stack([packed & 0xF, packed >> 4], axis=-1).reshape(packed.shape[0], 16)
+
+    for first, negative in ((1, 0), (3, 1)):
+        got = np.concatenate([codes[first, 1:16], codes[first + 1, 1:15]])
+        assert np.array_equal(np.abs(lut[got]), want), (negative, got)
+        assert np.array_equal(got >> 3, np.full(29, negative, dtype=got.dtype))
+
+    a = GOLDEN["fp4_anchor"]
+    assert codes[5, 1:9].tolist() == a["codes"]
+    assert codes[5, 9:11].tolist() == [GOLDEN["fp4_signed_zero"]["+0.0"],
+                                       GOLDEN["fp4_signed_zero"]["-0.0"]]
+    # the anchor bytes themselves: codes 0..7 starting at an even column
+    row = np.concatenate([lut[:8], [6.0], np.zeros(7)]).astype(np.float32)
+    qa = NVFP4QWeight.from_float(torch.from_numpy(np.stack([top, row])).cuda())
+    assert qa.weight_packed.cpu().numpy()[1, :4].tolist() == [h(b) for b in a["packed_bytes"]]
+
+    # far above the grid: saturates at +-6
+    sat = np.zeros((1, 16), dtype=np.float32)
+    sat[0, 0], sat[0, 1] = 1e6, -1e6
+    byte = int(NVFP4QWeight.from_float(torch.from_numpy(sat).cuda()).weight_packed[0, 0])
+    assert (byte & 0xF, byte >> 4) == (7, 15)
