@@ -26,6 +26,16 @@
 #ifndef OA_ADAM_NT_ST
 #define OA_ADAM_NT_ST 1
 #endif
+// The fp32 master is read as two 16-byte halves per lane, so one wave
+// instruction uses half of every 128-byte line it touches and the next one
+// the other half: a temporal load lets the second hit in cache (+2.6 % on a
+// 58.7 M-element tensor); the stores stay non-temporal (temporal: -4 %).
+#ifndef OA_ADAM_MASTER_LD_NT
+#define OA_ADAM_MASTER_LD_NT 0
+#endif
+#ifndef OA_ADAM_MASTER_ST_NT
+#define OA_ADAM_MASTER_ST_NT 1
+#endif
 
 namespace oa {
 namespace {
@@ -200,8 +210,13 @@ __device__ __forceinline__ void adam_tile(const AdamArgs& a, int64_t tile, bool 
       Vo[k] = ld(reinterpret_cast<const u32x4*>(a.v + e0));
       if (MODE == kFp32Master) {
         const float* mp = reinterpret_cast<const float*>(a.aux) + e0;
+#if OA_ADAM_MASTER_LD_NT
         Ma[k] = ld(reinterpret_cast<const f32x4*>(mp));
         Mb[k] = ld(reinterpret_cast<const f32x4*>(mp + 4));
+#else
+        Ma[k] = *reinterpret_cast<const f32x4*>(mp);
+        Mb[k] = *reinterpret_cast<const f32x4*>(mp + 4);
+#endif
       }
       if (MODE == kFp31 || MODE == kCustom)
         E[k] = ld(reinterpret_cast<const u32x4*>(
@@ -279,8 +294,13 @@ __device__ __forceinline__ void adam_tile(const AdamArgs& a, int64_t tile, bool 
     st(reinterpret_cast<u32x4*>(a.p + e0), Pn);
     if (MODE == kFp32Master) {
       float* mp = reinterpret_cast<float*>(a.aux) + e0;
+#if OA_ADAM_MASTER_ST_NT
       st(reinterpret_cast<f32x4*>(mp), Mlo);
       st(reinterpret_cast<f32x4*>(mp + 4), Mhi);
+#else
+      *reinterpret_cast<f32x4*>(mp) = Mlo;
+      *reinterpret_cast<f32x4*>(mp + 4) = Mhi;
+#endif
     }
     if (MODE == kFp31 || MODE == kCustom)
       st(reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.aux) + e0), En);
