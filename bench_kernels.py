@@ -2,9 +2,10 @@
 """Per-kernel throughput of everything on the optimizer path besides the fused
 AdamW launch that ``bench.py`` measures: gradient L2 norm, clip coefficient,
 the fused AdamW kernel with the clip coefficient folded in (fp31_master), and
-the eight weight codecs.  One JSON line per kernel.
+the eight weight codecs, and the fp32_master step of a quantised weight (fused
+with its re-encoding, and as the reference's two moves).  One JSON line per kernel.
 
-    python bench_kernels.py [--reps 20] [--only norm_large,norm_small,clip,adam,codecs]
+    python bench_kernels.py [--reps 20] [--only norm_large,norm_small,clip,adam,codecs,qat]
 
 Shapes: the offloaded parameters of a Llama-3-8B-shaped decoder for the norm
 and AdamW kernels, one 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
@@ -173,11 +174,58 @@ def bench_codecs(args, torch):
     line("dequant_nvfp4_kernel", wl + ", group 16", n * 2.5 + n // 16, us)
 
 
+def bench_qat_step(args, torch):
+    """fp32_master AdamW on a quantised 4096 x 14336 weight, then its payload
+    re-encoded from the new master: one fused launch (oa_adam_requant_*) against
+    the two moves of the reference (step with the gradient buffer as bf16 sink,
+    then copy_(master))."""
+    from offload_adam_amd.kernels import adam_step_fp32_master
+    from offload_adam_amd.qweight import Int4QWeight, Int8QWeight, NF4QWeight, NVFP4QWeight
+
+    n = ROWS * COLS
+    slots = 4
+    bf16 = torch.bfloat16
+    hyp = (1e-4, 0.01, 0.9, 0.999, 1e-8, 10)
+
+    def states():
+        w = outlier_weight(torch, 0, bf16)
+        return {"grad": (torch.randn(ROWS, COLS, device="cuda") * 5e-3).to(bf16),
+                "exp_avg": (torch.randn(ROWS, COLS, device="cuda") * 1e-4).to(bf16),
+                "exp_avg_sq": (torch.randn(ROWS, COLS, device="cuda") * 1e-3).square().to(bf16),
+                "master_params": w.float()}
+
+    sts = [states() for _ in range(slots)]
+    formats = (("int8", Int8QWeight, {}, 1 + 2 / COLS),
+               ("int4", Int4QWeight, {"group_size": 128}, 0.5 + 2 / 128),
+               ("nf4", NF4QWeight, {"blocksize": 64}, 0.5 + 4 / 64),
+               ("nvfp4", NVFP4QWeight, {}, 0.5 + 1 / 16))
+    for name, cls, kw, payload_bpe in formats:
+        qws = [cls.from_float(outlier_weight(torch, s, bf16), **kw) for s in range(slots)]
+        wl = f"4096x14336 {name} weight, fp32 master, bf16 moments"
+        us = timed(lambda i: adam_step_fp32_master(qws[i % slots], sts[i % slots], *hyp,
+                                                   decoupled_weight_decay=True),
+                   args.reps, torch)
+        # NVFP4 reads the stored master once more for the encode launch
+        extra = 4 if name == "nvfp4" else 0
+        line(f"adam fp32_master + requant {name}, fused", wl, n * (18 + extra + payload_bpe), us)
+
+        def two_moves(i):
+            st = sts[i % slots]
+            adam_step_fp32_master(st["grad"], st, *hyp, decoupled_weight_decay=True)
+            qws[i % slots].copy_(st["master_params"])
+
+        us2 = timed(two_moves, args.reps, torch)
+        line(f"adam fp32_master + requant {name}, two moves", wl,
+             n * (20 + 4 + extra + payload_bpe), us2, fused_speedup=round(us2 / us, 3))
+        del qws
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=40)
-    ap.add_argument("--only", default="norm_large,norm_small,clip,adam,codecs",
-                    help="comma-separated subset of: norm_large, norm_small, clip, adam, codecs")
+    ap.add_argument("--only", default="norm_large,norm_small,clip,adam,codecs,qat",
+                    help="comma-separated subset of: norm_large, norm_small, clip, adam, codecs, "
+                         "qat")
     args = ap.parse_args()
 
     import torch
@@ -196,6 +244,8 @@ def main():
         bench_adam_clip(args, torch)
     if "codecs" in todo:
         bench_codecs(args, torch)
+    if "qat" in todo:
+        bench_qat_step(args, torch)
 
 
 if __name__ == "__main__":

@@ -77,7 +77,9 @@ const char* oa_error_string(int code);
  * without its trailing device-wide synchronize.
  *   param_out  bf16[n], write-only: bf16_rne(master)   (may alias `grad`; the
  *              reference passes the grad buffer as a sink for quantised
- *              params, offload_adam.py:427-431)
+ *              params, offload_adam.py:427-431).  NULL: no bf16 copy is written
+ *              (18 instead of 20 bytes per element), for callers that re-encode
+ *              the parameter from `master` anyway.
  *   master     f32[n], read-write */
 int oa_adam_fp32_master(void* param_out, const void* grad, void* exp_avg,
                         void* exp_avg_sq, void* master, int64_t n, float lr,
@@ -272,6 +274,45 @@ int oa_dequant_nvfp4(const void* packed, const void* block_scale,
                      const void* global_scale, int64_t rows, int64_t cols,
                      void* out, int out_dtype, int64_t out_row_stride,
                      void* stream);
+
+/* fp32_master AdamW step and re-encoding of a quantised weight in one pass.
+ * Replaces, for a quantised parameter, the pair the reference runs per step:
+ * adam_step_fp32_master with the gradient buffer as a dummy bf16 sink
+ * (src/offload_adam/offload_adam.py:427-442, src/offload_adam/adam.py:139-149)
+ * followed by `p.data.copy_(master)` -> _quantize_*_triton
+ * (offload_adam.py:443-444; int8.py:430-442, int4.py:499-515, nf4.py:604-616,
+ * nvfp4.py:952-966).  The encoder's read of each element is the AdamW update of
+ * that element: grad/exp_avg/exp_avg_sq (bf16) and master (f32), all
+ * [rows*cols] contiguous, are updated exactly as oa_adam_fp32_master does
+ * (clip_coef as there; no bf16 copy of the master is written) and the payload is
+ * written exactly as oa_quant_* would write it from the new master.
+ * 18 + payload bytes per element instead of 20 + 4 + payload.
+ * Requirements (else OA_EINVAL / OA_EALIGN, and the caller runs the two calls
+ * separately): cols % 8 == 0, 16-byte aligned arrays; int4: group a power of two
+ * <= 512; nf4: block/8 a power of two, block <= 512; nvfp4: cols % 16 == 0
+ * (three launches: step + per-block amax, global scale, encode from master). */
+int oa_adam_requant_int8(const void* grad, void* exp_avg, void* exp_avg_sq,
+                         void* master, int64_t rows, int64_t cols, float lr,
+                         float weight_decay, float beta1_hat, float beta2_hat,
+                         float eps, int decoupled, const void* clip_coef, void* q,
+                         void* scales, int scale_dtype, void* stream);
+int oa_adam_requant_int4(const void* grad, void* exp_avg, void* exp_avg_sq,
+                         void* master, int64_t rows, int64_t cols, float lr,
+                         float weight_decay, float beta1_hat, float beta2_hat,
+                         float eps, int decoupled, const void* clip_coef,
+                         int64_t group, void* qweight, void* scales,
+                         int scale_dtype, void* stream);
+int oa_adam_requant_nf4(const void* grad, void* exp_avg, void* exp_avg_sq,
+                        void* master, int64_t rows, int64_t cols, float lr,
+                        float weight_decay, float beta1_hat, float beta2_hat,
+                        float eps, int decoupled, const void* clip_coef,
+                        int64_t block, void* packed, void* absmax, void* stream);
+int oa_adam_requant_nvfp4(const void* grad, void* exp_avg, void* exp_avg_sq,
+                          void* master, int64_t rows, int64_t cols, float lr,
+                          float weight_decay, float beta1_hat, float beta2_hat,
+                          float eps, int decoupled, const void* clip_coef,
+                          void* packed, void* block_scale, void* global_scale,
+                          void* workspace, void* stream);
 
 /* ------------------------------------------------------------------------
  * D. Pinned host memory and host<->device streaming.

@@ -93,6 +93,24 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p],
     ),
+    "oa_adam_requant_int8": (
+        c_int,
+        [c_void_p] * 4 + [c_int64] + _ADAM_TAIL + [c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+    ),
+    "oa_adam_requant_int4": (
+        c_int,
+        [c_void_p] * 4 + [c_int64] + _ADAM_TAIL
+        + [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p],
+    ),
+    "oa_adam_requant_nf4": (
+        c_int,
+        [c_void_p] * 4 + [c_int64] + _ADAM_TAIL + [c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
+    "oa_adam_requant_nvfp4": (
+        c_int,
+        [c_void_p] * 4 + [c_int64] + _ADAM_TAIL
+        + [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
     "oa_pinned_alloc": (
         c_int,
         [c_size_t, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int)],

@@ -142,10 +142,13 @@ class Adam(Optimizer):
                     batch_steps.append(state["step"])
                     continue
                 # The kernel writes a bf16 copy of the master through its first
-                # argument; for a quantised weight that goes to the grad buffer
-                # (a sink of matching shape) and the payload is re-encoded below.
+                # argument.  Given a quantised weight the fp32_master step
+                # function re-encodes the payload from the new master in the same
+                # pass; any other step function gets the grad buffer as a sink of
+                # matching shape and the payload is re-encoded below.
+                fused = quant and self.mode == "fp32_master"
                 self.step_fn(
-                    grad if quant else p.data,
+                    grad if quant and not fused else p.data,
                     tensors,
                     group["lr"],
                     group["weight_decay"],
@@ -156,8 +159,9 @@ class Adam(Optimizer):
                     decoupled_weight_decay=self.decoupled_weight_decay,
                 )
                 if quant:
-                    p.data.copy_(state["master_params"])
-                    p.grad = None  # it now holds the bf16 master, not a gradient
+                    if not fused:
+                        p.data.copy_(state["master_params"])
+                    p.grad = None  # as the reference leaves it (there it held the sink)
             if batch_p:
                 adam_step_multi(
                     self.mode,

@@ -113,15 +113,7 @@ __device__ __forceinline__ void adam_elem(uint32_t& pb, uint32_t gb, float& m,
     M = __uint_as_float((pb << 16) + (uint32_t)e);
   }
 
-  if (DEC) {
-    M = M - a.lr_wd * M;
-  } else {
-    g = g + a.wd * M;
-  }
-  m = m + a.omb1 * (g - m);
-  v = v + a.omb2 * (g * g - v);
-  const float denom = sqrtf(v) + a.eps;
-  M = M - (a.lr * m) / denom;
+  adam_core(M, g, m, v, DEC, a.lr, a.wd, a.lr_wd, a.omb1, a.omb2, a.eps);
 
   const uint32_t x = __float_as_uint(M);
   if (MODE == kFp32Master) {
@@ -162,7 +154,7 @@ __device__ __forceinline__ void adam_scalar(int64_t i, float clip,
   if (MODE == kStochastic) r16 = rand16_of<RNG>(i, a);
   adam_elem<MODE, DEC, CLIP>(pb, gb, m, v, aux, r16, clip, a);
   if (MODE == kFp32Master) pb = f32_to_bf16_1(__uint_as_float(aux));
-  a.p[i] = (uint16_t)pb;
+  if (MODE != kFp32Master || a.p) a.p[i] = (uint16_t)pb;  // fp32_master: the bf16 copy is optional
   a.m[i] = (uint16_t)f32_to_bf16_1(m);
   a.v[i] = (uint16_t)f32_to_bf16_1(v);
   if (MODE == kFp32Master) reinterpret_cast<uint32_t*>(a.aux)[i] = aux;
@@ -291,7 +283,7 @@ __device__ __forceinline__ void adam_tile(const AdamArgs& a, int64_t tile, bool 
 
     st(reinterpret_cast<u32x4*>(a.m + e0), Mn);
     st(reinterpret_cast<u32x4*>(a.v + e0), Vn);
-    st(reinterpret_cast<u32x4*>(a.p + e0), Pn);
+    if (MODE != kFp32Master || a.p) st(reinterpret_cast<u32x4*>(a.p + e0), Pn);
     if (MODE == kFp32Master) {
       float* mp = reinterpret_cast<float*>(a.aux) + e0;
 #if OA_ADAM_MASTER_ST_NT
@@ -311,32 +303,6 @@ __device__ __forceinline__ void adam_tile(const AdamArgs& a, int64_t tile, bool 
     const int64_t i = (n_groups << 3) + threadIdx.x;
     if (i < a.n) adam_scalar<MODE, DEC, CLIP, RNG>(i, clip, a);
   }
-}
-
-// Workgroup -> tile.  The dispatcher deals consecutive workgroups to the 8 XCDs
-// round-robin (workgroup b runs on XCD b % 8), each with its own L2.  With
-// tile = b every XCD touches every 8th tile of every array; mapping so that an
-// XCD owns runs of OA_ADAM_XCD_CHUNK consecutive tiles gives each L2 and the
-// memory channels behind it longer sequential streams (measured on a 4-read /
-// 3-write stream kernel of this shape: +3 % at 15 GB, +10 % at 0.8 GB per
-// launch).  The map is a bijection on [0, round_up(tiles, 8 * chunk)); grids are
-// padded to that size and surplus workgroups exit.
-#ifndef OA_ADAM_XCD_CHUNK
-#define OA_ADAM_XCD_CHUNK 64
-#endif
-constexpr uint32_t kXcds = 8;
-constexpr uint32_t kXcdChunk = OA_ADAM_XCD_CHUNK;
-
-__device__ __forceinline__ uint32_t xcd_tile(uint32_t b) {
-  if (kXcdChunk == 0) return b;
-  const uint32_t x = b % kXcds, j = b / kXcds;
-  const uint32_t c = j / kXcdChunk, r = j % kXcdChunk;
-  return (c * kXcds + x) * kXcdChunk + r;
-}
-inline uint32_t xcd_grid(uint32_t tiles) {
-  if (kXcdChunk == 0) return tiles;
-  const uint32_t q = kXcds * kXcdChunk;
-  return (tiles + q - 1) / q * q;
 }
 
 template <int MODE, bool DEC, bool CLIP, int RNG>
@@ -430,10 +396,10 @@ int dispatch_flags(const AdamArgs& a, bool dec, bool vec, hipStream_t s) {
 // Argument checks shared by the four entry points.  Returns 0, or an OA_E*.
 int check_common(const void* p, const void* g, const void* m, const void* v,
                  const void* aux, bool has_aux, size_t aux_align, int64_t n,
-                 const void* clip, bool p_may_alias_g) {
+                 const void* clip, bool p_may_alias_g, bool p_optional = false) {
   if (n < 0) return OA_EINVAL;
   if (n == 0) return 0;
-  if (!p || !g || !m || !v || (has_aux && !aux)) return OA_EINVAL;
+  if ((!p && !p_optional) || !g || !m || !v || (has_aux && !aux)) return OA_EINVAL;
   if (!aligned_to(p, 2) || !aligned_to(g, 2) || !aligned_to(m, 2) ||
       !aligned_to(v, 2) || (has_aux && !aligned_to(aux, aux_align)) ||
       (clip && !aligned_to(clip, 2)))
@@ -494,7 +460,7 @@ extern "C" int oa_adam_fp32_master(void* param_out, const void* grad, void* exp_
                                    float beta2_hat, float eps, int decoupled,
                                    const void* clip_coef, void* stream) {
   int rc = check_common(param_out, grad, exp_avg, exp_avg_sq, master, true, 4, n,
-                        clip_coef, /*p_may_alias_g=*/true);
+                        clip_coef, /*p_may_alias_g=*/true, /*p_optional=*/true);
   if (rc != 0 || n == 0) return rc;
   AdamArgs a = make_args(param_out, grad, exp_avg, exp_avg_sq, master, n, lr,
                          weight_decay, beta1_hat, beta2_hat, eps, clip_coef);

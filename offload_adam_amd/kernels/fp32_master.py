@@ -31,10 +31,31 @@ def adam_step_fp32_master(
     is accepted and ignored.  Unlike the reference it does not synchronize the
     device.  ``clip_coef`` (optional 0-dim bf16 GPU tensor) scales the gradient
     inside the kernel with the rounding of ``grad.mul_(clip_coef)``.
+
+    Two further forms of ``params``: ``None`` writes no bf16 copy at all, and a
+    quantised weight (``QWeightBase``) gets its payload re-encoded from the new
+    master - what the reference does with the gradient buffer as a throw-away
+    sink followed by ``p.data.copy_(master)`` (offload_adam.py:427-444) - in
+    the same pass when the layout allows, in a second launch otherwise.
     """
-    n = params.numel()
-    dev = params.device
-    _common.check_tensor(params, "params", torch.bfloat16, n, dev)
+    from ..qweight.base import QWeightBase
+
+    if isinstance(params, QWeightBase):
+        from .qat_step import adam_step_requant
+
+        if params.is_cuda and adam_step_requant(
+                params, states, lr, weight_decay, beta1, beta2, eps, step,
+                decoupled_weight_decay, clip_coef):
+            return
+        adam_step_fp32_master(None, states, lr, weight_decay, beta1, beta2, eps, step,
+                              decoupled_weight_decay, clip_coef=clip_coef)
+        params.copy_(states["master_params"])
+        return
+    master = states["master_params"]
+    n = master.numel()
+    dev = master.device
+    if params is not None:
+        _common.check_tensor(params, "params", torch.bfloat16, n, dev)
     _common.check_tensor(states["grad"], "states['grad']", torch.bfloat16, n, dev)
     _common.check_tensor(states["exp_avg"], "states['exp_avg']", torch.bfloat16, n, dev)
     _common.check_tensor(
@@ -48,7 +69,7 @@ def adam_step_fp32_master(
         return
     _common.launch(
         "oa_adam_fp32_master",
-        params,
+        master,
         [
             _lib.ptr(params),
             _lib.ptr(states["grad"]),
@@ -57,7 +78,7 @@ def adam_step_fp32_master(
             _lib.ptr(states["master_params"]),
         ],
         _common.scalar_args(
-            params, lr, weight_decay, beta1, beta2, eps, step, decoupled_weight_decay
+            master, lr, weight_decay, beta1, beta2, eps, step, decoupled_weight_decay
         )
         + [_lib.ptr(clip_coef)],
     )

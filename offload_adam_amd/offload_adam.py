@@ -556,10 +556,13 @@ class OffloadAdam(Optimizer):
         quant = p in self._quant_params
         if quant:
             self._maybe_warn_quant_master(state)
-        # A quantised weight cannot take the kernel's bf16 write-back: it goes to
-        # the gradient buffer (a sink) and the payload is re-encoded from the master.
+        # A quantised weight cannot take the kernel's bf16 write-back.  The
+        # fp32_master step function re-encodes the payload from the new master
+        # itself (one fused pass); any other step function writes its bf16 copy
+        # to the gradient buffer (a sink) and the payload is re-encoded after it.
+        fused = quant and self.mode == "fp32_master"
         self.step_fn(
-            tensors["grad"] if quant else p.data,
+            tensors["grad"] if quant and not fused else p.data,
             tensors,
             group["lr"],
             group["weight_decay"],
@@ -570,7 +573,7 @@ class OffloadAdam(Optimizer):
             decoupled_weight_decay=self.decoupled_weight_decay,
             clip_coef=clip_coef,
         )
-        if quant:
+        if quant and not fused:
             p.data.copy_(tensors["master_params"])
 
     def _step_offload(self, p, group, clip_coef=None):
