@@ -332,3 +332,96 @@ def test_argument_errors():
     rc = lib.oa_adam_fp32_master(_lib.ptr(p), _lib.ptr(st["grad"]), _lib.ptr(m), _lib.ptr(m),
                                  _lib.ptr(st["master_params"]), 16, 0, 0, 0, 0, 0, 0, None, None)
     assert rc == -4
+
+
+def _llama_1b_shapes():
+    """The 201 parameter tensors of BASELINE config 1 (hidden 2048, MLP 5632, 22
+    layers, 32 query / 4 key-value heads of 64, vocabulary 32000, untied)."""
+    h, inter, layers, kv, vocab = 2048, 5632, 22, 4 * 64, 32000
+    shapes = [(vocab, h)]
+    for _ in range(layers):
+        shapes += [(h,), (h, h), (kv, h), (kv, h), (h, h), (h,), (inter, h), (inter, h), (h, inter)]
+    shapes += [(h,), (vocab, h)]
+    return shapes
+
+
+def test_config1_full_set(oracle):
+    """BASELINE config 1 at full size: 201 tensors, 1,100,048,384 elements,
+    stochastic rounding, one multi-tensor step (6 launches).
+
+    * one tensor of every distinct size (82 M elements) is compared bit for bit
+      with the C oracle;
+    * every tensor is checked through size-independent properties evaluated with
+      plain fp32 torch ops on the GPU: the stored moments are exactly
+      bf16_rne(m + (1-b1)(g-m)) and bf16_rne(v + (1-b2)(g*g-v)); the stored
+      parameter is the fp32 result M' truncated to bf16 or one step above in
+      magnitude (M' taken within 1 fp32 ulp: torch's own sqrt and divide are
+      not promised correctly rounded); and over the whole set the number of
+      round-ups matches the sum of the round-up probabilities frac/65536
+      (unbiasedness) within 6 standard deviations."""
+    from offload_adam_amd.kernels import adam_step_multi
+
+    shapes = _llama_1b_shapes()
+    assert len(shapes) == 201 and sum(int(np.prod(s)) for s in shapes) == 1_100_048_384
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    params, states, seeds = [], [], []
+    for i, shape in enumerate(shapes):
+        n = int(np.prod(shape))
+        params.append((torch.randn(n, device="cuda", generator=gen) * 0.02).to(torch.bfloat16))
+        states.append({
+            "grad": (torch.randn(n, device="cuda", generator=gen) * 1e-3).to(torch.bfloat16),
+            "exp_avg": (torch.randn(n, device="cuda", generator=gen) * 1e-4).to(torch.bfloat16),
+            "exp_avg_sq": (torch.randn(n, device="cuda", generator=gen) * 1e-3).square()
+            .to(torch.bfloat16),
+        })
+        seeds.append(0x5EED0000 + i)
+    old = [(p.clone(), st["exp_avg"].clone(), st["exp_avg_sq"].clone())
+           for p, st in zip(params, states)]
+    first_of_size = {}
+    for i, p in enumerate(params):
+        first_of_size.setdefault(p.numel(), i)
+    refs = {}
+    for i in first_of_size.values():
+        refs[i] = _oracle_step(oracle, "stochastic_rounding", params[i], states[i], True, None,
+                               seed=seeds[i], layout=1)
+    assert sum(params[i].numel() for i in refs) > 80_000_000 and len(refs) == 5
+
+    adam_step_multi("stochastic_rounding", params, states, HYP["lr"], HYP["weight_decay"],
+                    HYP["beta1"], HYP["beta2"], HYP["eps"], HYP["step"],
+                    decoupled_weight_decay=True, seeds=seeds, rng="x8")
+    torch.cuda.synchronize()
+    for i, ref in refs.items():
+        _assert_equal("stochastic_rounding", params[i], states[i], ref, f"config 1 tensor {i}")
+
+    b1h, b2h = oracle.folded_betas(HYP["beta1"], HYP["beta2"], HYP["step"])
+    f32 = np.float32
+    omb1, omb2 = float(f32(1) - f32(b1h)), float(f32(1) - f32(b2h))
+    lr, eps = float(f32(HYP["lr"])), float(f32(HYP["eps"]))
+    lr_wd = float(f32(HYP["lr"]) * f32(HYP["weight_decay"]))
+    ups = 0.0
+    expected_ups = 0.0
+    variance = 0.0
+    for i, (p, st) in enumerate(zip(params, states)):
+        p0, m0, v0 = (t.float() for t in old[i])
+        g = st["grad"].float()
+        m = m0 + omb1 * (g - m0)
+        v = v0 + omb2 * (g * g - v0)
+        assert torch.equal(st["exp_avg"], m.to(torch.bfloat16)), f"tensor {i} exp_avg"
+        assert torch.equal(st["exp_avg_sq"], v.to(torch.bfloat16)), f"tensor {i} exp_avg_sq"
+        M = p0 - lr_wd * p0
+        M = M - (lr * m) / (torch.sqrt(v) + eps)
+        mb = M.view(torch.int32)
+        pb = p.view(torch.int16).to(torch.int32) << 16
+
+        def on_grid(b):
+            t = b & -0x10000
+            return (pb == t) | (pb == t + 0x10000)
+
+        ok = on_grid(mb) | on_grid(mb + 1) | on_grid(mb - 1)
+        assert bool(ok.all()), f"tensor {i}: {int((~ok).sum())} params off the two bf16 neighbours"
+        frac = (mb & 0xFFFF).double() / 65536.0
+        ups += float((pb != (mb & -0x10000)).double().sum())
+        expected_ups += float(frac.sum())
+        variance += float((frac * (1 - frac)).sum())
+        old[i] = None
+    assert abs(ups - expected_ups) < 6.0 * variance ** 0.5 + 1e3, (ups, expected_ups, variance)

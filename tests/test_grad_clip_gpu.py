@@ -132,3 +132,136 @@ def test_config2_norm_and_clip_flow(oracle):
     assert abs(total.item() - 3.0) < 0.05
     assert abs(coef.item() - 1.0 / 3.0) < 0.01
     assert bits(coef.reshape(1))[0] == oracle.clip_coef_bf16(bits(total.reshape(1))[0], 1.0)
+
+
+def _llama_8b_shapes():
+    """The 291 parameter tensors of BASELINE config 2 / 4 (hidden 4096, MLP 14336,
+    32 layers, 32 query / 8 key-value heads of 128, vocabulary 128256, untied)."""
+    h, inter, layers, kv, vocab = 4096, 14336, 32, 8 * 128, 128256
+    shapes = [(vocab, h)]
+    for _ in range(layers):
+        shapes += [(h,), (h, h), (kv, h), (kv, h), (h, h), (h,), (inter, h), (inter, h), (h, inter)]
+    shapes += [(h,), (vocab, h)]
+    return shapes
+
+
+def test_config2_full_set(oracle):
+    """BASELINE config 2 at full size, kernel legs on GPU-resident buffers: 291
+    tensors, 8,030,261,248 elements, fp31_master, gradients with a global norm of
+    about 3 clipped to max_grad_norm = 1 inside the AdamW kernel.
+
+    * every per-tensor norm within one bf16 ulp of torch.norm, the total within
+      one ulp of the fp64 value, the coefficient bit-exact given the total;
+    * one tensor of every size below 60 M elements and the first 4 M elements of
+      an embedding are compared bit for bit with the C oracle;
+    * every tensor through size-independent properties, in plain fp32 torch ops
+      on the GPU: moments exactly bf16_rne of the update computed from the
+      clipped gradient bf16_rne(g * coef); the (param, rounding_error) pair
+      reconstructs round_to_fp31(M') with M' taken within one fp32 ulp; the
+      param is exactly bf16_rne of that master; the error stays in
+      [-16384, 16384]."""
+    import numpy as np
+
+    from offload_adam_amd.grad_clip import clip_coef_, grad_norm_
+    from offload_adam_amd.kernels import adam_step_multi
+
+    shapes = _llama_8b_shapes()
+    numels = [int(np.prod(s)) for s in shapes]
+    total_n = sum(numels)
+    assert len(shapes) == 291 and total_n == 8_030_261_248
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    g_std = 3.0 / total_n ** 0.5
+
+    def draw(n, std):
+        return (torch.randn(n, device="cuda", generator=gen) * std).to(BF16)
+
+    grads = [draw(n, g_std) for n in numels]
+    norms = torch.zeros(len(grads), dtype=BF16, device="cuda")
+    for i, g in enumerate(grads):
+        grad_norm_(g, norms[i])
+    coef = torch.empty((), dtype=BF16, device="cuda")
+    total = torch.empty((), dtype=BF16, device="cuda")
+    clip_coef_(norms, 1.0, coef, total)
+    torch.cuda.synchronize()
+    norm_bits = bits(norms)
+    sumsq = 0.0
+    for i, g in enumerate(grads):
+        lib = torch.norm(g, 2.0)
+        assert _ulp_diff(norm_bits[i], bits(lib.reshape(1))[0]) <= 1, f"norm of tensor {i}"
+        sumsq += float(norms[i].double()) ** 2
+    want_total = torch.tensor(sumsq ** 0.5, dtype=torch.float64).to(BF16)
+    assert _ulp_diff(bits(total.reshape(1))[0], bits(want_total.reshape(1))[0]) <= 1
+    assert abs(total.item() - 3.0) < 0.05 and abs(coef.item() - 1.0 / 3.0) < 0.01
+    coef_bits = bits(coef.reshape(1))[0]
+    assert coef_bits == oracle.clip_coef_bf16(bits(total.reshape(1))[0], 1.0)
+
+    b1h, b2h = oracle.folded_betas(HYP["beta1"], HYP["beta2"], HYP["step"])
+    f32 = np.float32
+    omb1, omb2 = float(f32(1) - f32(b1h)), float(f32(1) - f32(b2h))
+    lr, eps = float(f32(HYP["lr"])), float(f32(HYP["eps"]))
+    lr_wd = float(f32(HYP["lr"]) * f32(HYP["weight_decay"]))
+    oracle_args = (HYP["lr"], HYP["weight_decay"], b1h, b2h, HYP["eps"], True)
+    sizes_checked = set()
+    chunk = 36  # tensors per launch of the multi-tensor kernel
+    for c0 in range(0, len(shapes), chunk):
+        idx = range(c0, min(c0 + chunk, len(shapes)))
+        params = [draw(numels[i], 0.02) for i in idx]
+        states = [{"grad": grads[i], "exp_avg": draw(numels[i], 1e-4),
+                   "exp_avg_sq": draw(numels[i], 1e-3).float().square().to(BF16),
+                   "rounding_error": torch.randint(-16384, 16385, (numels[i],), device="cuda",
+                                                   generator=gen, dtype=torch.int16)}
+                  for i in idx]
+        old = [(p.clone(), st["exp_avg"].clone(), st["exp_avg_sq"].clone(),
+                st["rounding_error"].clone()) for p, st in zip(params, states)]
+        # oracle on CPU copies taken before the step
+        refs = {}
+        for j, i in enumerate(idx):
+            n = numels[i]
+            take = n if n < 60_000_000 else 4_000_000
+            if (n, take) in sizes_checked:
+                continue
+            sizes_checked.add((n, take))
+            pb, gb = bits(params[j][:take]), bits(states[j]["grad"][:take])
+            mb, vb = bits(states[j]["exp_avg"][:take]), bits(states[j]["exp_avg_sq"][:take])
+            err = states[j]["rounding_error"][:take].cpu().numpy().copy()
+            oracle.adam_fp31_master(pb, gb, mb, vb, err, *oracle_args,
+                                    clip=np.array([coef_bits], dtype=np.uint16))
+            refs[j] = (take, pb, mb, vb, err)
+        adam_step_multi("fp31_master", params, states, HYP["lr"], HYP["weight_decay"],
+                        HYP["beta1"], HYP["beta2"], HYP["eps"], HYP["step"],
+                        decoupled_weight_decay=True, clip_coef=coef)
+        torch.cuda.synchronize()
+        for j, (take, pb, mb, vb, err) in refs.items():
+            ctx = f"config 2 tensor {c0 + j}"
+            assert np.array_equal(bits(params[j][:take]), pb), ctx + " param"
+            assert np.array_equal(bits(states[j]["exp_avg"][:take]), mb), ctx + " exp_avg"
+            assert np.array_equal(bits(states[j]["exp_avg_sq"][:take]), vb), ctx + " exp_avg_sq"
+            assert np.array_equal(states[j]["rounding_error"][:take].cpu().numpy(), err), ctx
+        for j, (p, st) in enumerate(zip(params, states)):
+            ctx = f"config 2 tensor {c0 + j}"
+            p0, m0, v0, e0 = old[j]
+            g = (st["grad"] * coef).float()
+            m0, v0 = m0.float(), v0.float()
+            m = m0 + omb1 * (g - m0)
+            v = v0 + omb2 * (g * g - v0)
+            assert torch.equal(st["exp_avg"], m.to(BF16)), ctx + " exp_avg"
+            assert torch.equal(st["exp_avg_sq"], v.to(BF16)), ctx + " exp_avg_sq"
+            M = ((p0.view(torch.int16).to(torch.int32) << 16) + (e0.to(torch.int32) << 1)
+                 ).view(torch.float32)
+            M = M - lr_wd * M
+            M = M - (lr * m) / (torch.sqrt(v) + eps)
+            # A random rounding error next to a param of exactly +-0 reconstructs to
+            # NaN bits, a state no run produces: those elements are left out.
+            fin = torch.isfinite(M)
+            assert int((~fin).sum()) <= 1 + p.numel() // 1_000_000, ctx + " non-finite masters"
+            b = M.view(torch.int32)
+            want = ((b >> 1) + (b & (b >> 1) & 1)) << 1
+            e1 = st["rounding_error"].to(torch.int32)
+            got = (p.view(torch.int16).to(torch.int32) << 16) + (e1 << 1)
+            assert int(((got - want).abs() * fin).max()) <= 2, ctx + " master"
+            same = p.view(torch.int16) == got.view(torch.float32).to(BF16).view(torch.int16)
+            assert bool((same | ~fin).all()), ctx + " param = bf16(master)"
+            assert int((e1.abs() * fin).max()) <= 16384, ctx + " error range"
+            old[j] = None
+        del params, states, old
+    assert len(sizes_checked) == 5

@@ -133,6 +133,13 @@ def test_zeros_pinned_invariants():
         assert free0 > 0
         t = zeros_pinned((1 << 20,), torch.float32, numa_node=0)
         assert not t.any() and t.is_pinned()
+        # a node the host does not have: the memory-policy call fails, nothing is allocated
+        with pytest.raises(OSError) as info:
+            zeros_pinned((4,), BF16, numa_node=1000)
+        assert info.value.errno > 0
+        # beyond what the node mask can name at all
+        with pytest.raises(RuntimeError):
+            zeros_pinned((4,), BF16, numa_node=5000)
     assert numa_node_free_bytes(10_000) is None
 
 
