@@ -5,7 +5,7 @@ the fused AdamW kernel with the clip coefficient folded in (fp31_master), and
 the eight weight codecs, and the fp32_master step of a quantised weight (fused
 with its re-encoding, and as the reference's two moves).  One JSON line per kernel.
 
-    python bench_kernels.py [--reps 20] [--only norm_large,norm_small,clip,adam,codecs,qat]
+    python bench_kernels.py [--reps 20] [--only norm_large,norm_small,clip,adam,codecs,qat,stream]
 
 Shapes: the offloaded parameters of a Llama-3-8B-shaped decoder for the norm
 and AdamW kernels, one 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
@@ -174,6 +174,37 @@ def bench_codecs(args, torch):
     line("dequant_nvfp4_kernel", wl + ", group 16", n * 2.5 + n // 16, us)
 
 
+def bench_stream_ceiling(args, torch):
+    """What a plain device-to-device copy reaches on this part: the runtime's own
+    copy kernel (``Tensor.copy_`` between two HBM buffers), reads + writes counted,
+    on buffers that rotate like the other sections'.  The yardstick the AdamW
+    kernels' 14-20 bytes per element are held against besides the 8 TB/s nameplate."""
+    from offload_adam_amd import grad_clip
+    from offload_adam_amd.offload_adam import _copy_by_kernel
+
+    # read-only: the gradient-norm kernel over 1 GiB
+    n = 512 << 20
+    gs = [torch.empty(n, dtype=torch.bfloat16, device="cuda").normal_(0, 1e-3) for _ in range(3)]
+    out = torch.zeros((), dtype=torch.bfloat16, device="cuda")
+    us = timed(lambda i: grad_clip.grad_norm_(gs[i % 3], out), args.reps, torch)
+    line("grad_norm_partial_kernel + grad_norm_final_kernel (read only)", "1024 MiB read", 2 * n, us)
+    del gs
+    for mib in (392, 1024):
+        n = mib << 20
+        slots = max(2, (3 << 30) // (2 * n) + 1)
+        src = [torch.empty(n, dtype=torch.uint8, device="cuda").random_() for _ in range(slots)]
+        dst = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(slots)]
+        wl = f"{mib} MiB read + {mib} MiB written"
+        us = timed(lambda i: dst[i % slots].copy_(src[i % slots]), args.reps, torch)
+        line("runtime device-to-device copy", wl, 2 * n, us)
+        stream = torch.cuda.current_stream()
+        for wgs in (1024, 4096):
+            us = timed(lambda i: _copy_by_kernel(dst[i % slots], src[i % slots], stream, wgs),
+                       args.reps, torch)
+            line(f"link_copy_kernel between HBM buffers, {wgs} workgroups", wl, 2 * n, us)
+        del src, dst
+
+
 def bench_qat_step(args, torch):
     """fp32_master AdamW on a quantised 4096 x 14336 weight, then its payload
     re-encoded from the new master: one fused launch (oa_adam_requant_*) against
@@ -223,9 +254,9 @@ def bench_qat_step(args, torch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=40)
-    ap.add_argument("--only", default="norm_large,norm_small,clip,adam,codecs,qat",
+    ap.add_argument("--only", default="norm_large,norm_small,clip,adam,codecs,qat,stream",
                     help="comma-separated subset of: norm_large, norm_small, clip, adam, codecs, "
-                         "qat")
+                         "qat, stream")
     args = ap.parse_args()
 
     import torch
@@ -246,6 +277,8 @@ def main():
         bench_codecs(args, torch)
     if "qat" in todo:
         bench_qat_step(args, torch)
+    if "stream" in todo:
+        bench_stream_ceiling(args, torch)
 
 
 if __name__ == "__main__":
