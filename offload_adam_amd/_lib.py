@@ -4,6 +4,7 @@ The library is loaded lazily on first use.  There is no fallback: if the
 shared object has not been built, every operator raises.
 """
 
+import contextlib
 import ctypes
 import os
 import threading
@@ -179,10 +180,30 @@ def check(code, what):
         raise RuntimeError(f"{what} failed with code {code}: {error_string(code)}")
 
 
-def current_stream_ptr():
+_NO_GUARD = contextlib.nullcontext()
+
+
+def device_guard(device):
+    """Context that makes ``device`` the current GPU; free when it already is
+    (``torch.cuda.device`` costs several microseconds per launch otherwise)."""
     import torch
 
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+    index = device.index
+    if index is None or index == torch._C._cuda_getDevice():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
+def current_stream_id():
+    """Raw handle (an int) of the calling thread's current stream on the current
+    GPU, without building a ``torch.cuda.Stream`` object."""
+    import torch
+
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
+
+
+def current_stream_ptr():
+    return c_void_p(current_stream_id())
 
 
 def ptr(t):

@@ -39,12 +39,12 @@ def grad_norm_(grad, out):
     if not grad.is_contiguous() or out.numel() != 1:
         raise ValueError("grad must be contiguous and out must hold one element")
     lib = _lib.load()
-    with torch.cuda.device(grad.device):
-        stream = torch.cuda.current_stream()
-        ws = _workspace(grad.device, stream.cuda_stream)
+    with _lib.device_guard(grad.device):
+        stream = _lib.current_stream_id()
+        ws = _workspace(grad.device, stream)
         code = lib.oa_grad_norm_bf16(
             _lib.ptr(grad), c_int64(grad.numel()), _lib.ptr(out), None, _lib.ptr(ws),
-            _lib.c_void_p(stream.cuda_stream),
+            _lib.c_void_p(stream),
         )
     _lib.check(code, "oa_grad_norm_bf16")
     return out
@@ -68,7 +68,7 @@ def clip_coef_(norms, max_grad_norm, coef_out, total_out=None):
     if total_out is not None and (total_out.dtype != torch.bfloat16 or total_out.numel() != 1):
         raise TypeError("total_out must be one bfloat16 element")
     lib = _lib.load()
-    with torch.cuda.device(norms.device):
+    with _lib.device_guard(norms.device):
         code = lib.oa_clip_coef_bf16(
             _lib.ptr(norms), c_int64(norms.numel()), c_float(max_grad_norm),
             _lib.ptr(total_out), _lib.ptr(coef_out), _lib.current_stream_ptr(),

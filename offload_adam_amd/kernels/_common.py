@@ -52,6 +52,6 @@ def scalar_args(params, lr, weight_decay, beta1, beta2, eps, step, decoupled):
 def launch(fn_name, params, ptr_args, tail_args):
     """Call an entry point on ``params``' device and current stream."""
     lib = _lib.load()
-    with torch.cuda.device(params.device):
+    with _lib.device_guard(params.device):
         code = getattr(lib, fn_name)(*ptr_args, *tail_args, _lib.current_stream_ptr())
     _lib.check(code, fn_name)

@@ -112,7 +112,7 @@ def adam_step_multi(
         return c_void_p(a.ctypes.data) if a is not None else c_void_p(None)
 
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         code = lib.oa_adam_multi(
             c_int(MODE_CODES[mode]), c_int(count), addr(p_tab), addr(g_tab), addr(m_tab),
             addr(v_tab), addr(a_tab), addr(n_tab), addr(b1), addr(b2), addr(seed_tab),

@@ -51,9 +51,8 @@ def _plan(qw):
         if cols % 16 != 0:
             return None
         payload = (qw.weight_packed, qw.block_scale_fp8, qw.global_scale)
-        with torch.cuda.device(qw.weight_packed.device):
-            ws = _codec_ops._amax_workspace(qw.weight_packed.device,
-                                            torch.cuda.current_stream().cuda_stream)
+        with _lib.device_guard(qw.weight_packed.device):
+            ws = _codec_ops._amax_workspace(qw.weight_packed.device, _lib.current_stream_id())
         tail = [_lib.ptr(qw.weight_packed), _lib.ptr(qw.block_scale_fp8),
                 _lib.ptr(qw.global_scale), _lib.ptr(ws)]
         name = "oa_adam_requant_nvfp4"
@@ -90,7 +89,7 @@ def adam_step_requant(qweight, states, lr, weight_decay, beta1, beta2, eps, step
     rows, cols = qweight.shape
     b1h, b2h = _common.folded_betas(beta1, beta2, step)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         code = getattr(lib, name)(
             _lib.ptr(states["grad"]), _lib.ptr(states["exp_avg"]), _lib.ptr(states["exp_avg_sq"]),
             _lib.ptr(master), c_int64(rows), c_int64(cols), c_float(lr), c_float(weight_decay),

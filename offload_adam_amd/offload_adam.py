@@ -328,6 +328,7 @@ class OffloadAdam(Optimizer):
         self.device_states = {}
         self.h2d_events = {}
         self.d2h_events = {}
+        self._compute_streams = {}  # raw stream handle -> torch.cuda.Stream
         self.transfer_stream_report = None
         if self._offload_params:
             self._check_copy_engines()
@@ -484,8 +485,18 @@ class OffloadAdam(Optimizer):
     def _host_view(self, p, name):
         return self.state[p][name]
 
+    def _compute_stream(self):
+        """The calling thread's current stream as a ``torch.cuda.Stream``; the
+        objects are kept per raw handle (building one costs ~3 us per call and a
+        hook needs it three times)."""
+        raw = _lib.current_stream_id()
+        stream = self._compute_streams.get(raw)
+        if stream is None:
+            stream = self._compute_streams[raw] = torch.cuda.current_stream()
+        return stream
+
     def _issue_h2d(self, p, keys):
-        compute = torch.cuda.current_stream()
+        compute = self._compute_stream()
         dev = self.device_states[p]
         if p in self.d2h_events:
             self.h2d_stream.wait_event(self.d2h_events[p])
@@ -498,7 +509,7 @@ class OffloadAdam(Optimizer):
         self.h2d_events[p] = self.h2d_stream.record_event()
 
     def _issue_d2h(self, p, keys):
-        compute = torch.cuda.current_stream()
+        compute = self._compute_stream()
         dev = self.device_states[p]
         self.d2h_stream.wait_stream(compute)
         for key in keys:
@@ -522,7 +533,7 @@ class OffloadAdam(Optimizer):
         if missing:
             self._issue_h2d(p, missing)
         if p in self.h2d_events:
-            torch.cuda.current_stream().wait_event(self.h2d_events[p])
+            self._compute_stream().wait_event(self.h2d_events[p])
 
     # ------------------------------------------------- per-parameter operations
 

@@ -45,7 +45,7 @@ def _payload(t, name, dtype, shape):
 
 def _call(name, device, *args):
     lib = _lib.load()
-    with torch.cuda.device(device):
+    with _lib.device_guard(device):
         code = getattr(lib, name)(*args, _lib.current_stream_ptr())
     _lib.check(code, name)
 
@@ -137,8 +137,8 @@ def quantize_nvfp4_into(src, packed, block_scale_fp8, global_scale):
     _payload(packed, "weight_packed", torch.uint8, (rows, cols // 2))
     _payload(block_scale_fp8, "block_scale_fp8", torch.float8_e4m3fn, (rows, cols // 16))
     _payload(global_scale, "global_scale", torch.float32, ())
-    with torch.cuda.device(src.device):
-        ws = _amax_workspace(src.device, torch.cuda.current_stream().cuda_stream)
+    with _lib.device_guard(src.device):
+        ws = _amax_workspace(src.device, _lib.current_stream_id())
     _call("oa_quant_nvfp4", src.device, _lib.ptr(src), c_int(_lib.dtype_code(src.dtype)),
           c_int64(stride), c_int64(rows), c_int64(cols), _lib.ptr(packed),
           _lib.ptr(block_scale_fp8), _lib.ptr(global_scale), _lib.ptr(ws))

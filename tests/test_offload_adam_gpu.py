@@ -154,6 +154,7 @@ def test_pinned_memory_is_released():
         freed.append(ptr.value if hasattr(ptr, "value") else ptr)
         return real(ptr)
 
+    gc.collect()  # buffers other tests left behind go now, not while this one watches
     lib.oa_pinned_free = spy
     try:
         t = pinned_alloc.zeros_pinned((1 << 20,), torch.float32, numa_node=None)
@@ -161,12 +162,12 @@ def test_pinned_memory_is_released():
         view = t[10:20]
         del t
         gc.collect()
-        assert freed == []  # a surviving view keeps the pages alive
+        assert ptr not in freed  # a surviving view keeps the pages alive
         view.fill_(3.0)
         assert view.sum().item() == 30.0
         del view
         gc.collect()
-        assert freed == [ptr]  # released exactly once, when the last view died
+        assert freed.count(ptr) == 1  # released exactly once, when the last view died
     finally:
         lib.oa_pinned_free = real
 
