@@ -886,5 +886,76 @@ class OffloadAdam(Optimizer):
         raise NotImplementedError(
             "OffloadAdam.load_state_dict is not supported: the default "
             "Optimizer.load_state_dict would move pinned-host state to GPU and cast fp32 "
-            "master to bf16, defeating the offload contract. File an issue if resume is needed."
+            "master to bf16, defeating the offload contract. Use load_offloaded_state_dict "
+            "to resume."
         )
+
+    @torch.no_grad()
+    def load_offloaded_state_dict(self, state_dict):
+        """Resume from ``state_dict()`` of an ``OffloadAdam`` over the same
+        parameters (same order, shapes, mode and clipping setting).
+
+        The reference has no resume path (``load_state_dict`` raises there as it
+        does here, src/offload_adam/offload_adam.py:672-678).  This copies the saved
+        values *into this optimizer's own buffers*: offloaded states stay in their
+        pinned host allocations in their own dtypes (fp32 masters stay fp32), the
+        states of the small GPU-resident parameters stay on the GPU, and nothing is
+        re-allocated.  ``lr``, ``betas``, ``eps`` and ``weight_decay`` are taken
+        from the saved param group.  Model weights are not part of it: load the
+        model's own ``state_dict`` first.
+
+        Call it at a step boundary.  Partial gradient sums of an unfinished
+        accumulation window travel with the state (``grad`` / ``host_grad_valid``)
+        unless the optimizer was built with ``offload_grads=False``, whose running
+        sums never reach the state dict.
+        """
+        saved_groups = state_dict["param_groups"]
+        saved_state = state_dict["state"]
+        if len(saved_groups) != len(self.param_groups):
+            raise ValueError(
+                f"saved state has {len(saved_groups)} param groups, this optimizer "
+                f"{len(self.param_groups)}")
+        pairs = []
+        for group, saved in zip(self.param_groups, saved_groups):
+            if len(saved["params"]) != len(group["params"]):
+                raise ValueError("a saved param group has a different number of parameters")
+            pairs.extend(zip(saved["params"], group["params"]))
+        # validate everything before the first byte moves
+        for key, p in pairs:
+            if key not in saved_state:
+                raise ValueError(f"saved state has no entry for parameter {key}")
+            mine, theirs = self.state[p], saved_state[key]
+            if set(mine) != set(theirs):
+                raise ValueError(
+                    f"parameter {key}: saved keys {sorted(theirs)} do not match this "
+                    f"optimizer's {sorted(mine)} (different mode, clipping or threshold?)")
+            for name, value in mine.items():
+                other = theirs[name]
+                if isinstance(value, torch.Tensor) != isinstance(other, torch.Tensor):
+                    raise ValueError(f"parameter {key}: '{name}' changes kind")
+                if isinstance(value, torch.Tensor) and (
+                        value.shape != other.shape or value.dtype != other.dtype):
+                    raise ValueError(
+                        f"parameter {key}: '{name}' is {tuple(other.shape)} {other.dtype} in the "
+                        f"saved state, {tuple(value.shape)} {value.dtype} here")
+        # nothing may be in flight or staged while the buffers are rewritten
+        torch.cuda.synchronize()
+        for dev in self.device_states.values():
+            for name in dev:
+                dev[name] = None
+        self.h2d_events.clear()
+        self.d2h_events.clear()
+        self._bw_cursor = -1
+        self._bw_issued_upto = 0
+        for key, p in pairs:
+            mine, theirs = self.state[p], saved_state[key]
+            for name, value in mine.items():
+                if isinstance(value, torch.Tensor):
+                    value.copy_(theirs[name])
+                else:
+                    mine[name] = theirs[name]
+        for group, saved in zip(self.param_groups, saved_groups):
+            for name, value in saved.items():
+                if name != "params":
+                    group[name] = value
+        torch.cuda.synchronize()

@@ -465,6 +465,90 @@ def test_adam_state_dict_round_trip_keeps_fp32_master():
         assert opt2.state[p2]["step"] == 1
 
 
+@pytest.mark.parametrize("mode", ["fp32_master", "fp31_master", "stochastic_rounding"])
+@pytest.mark.parametrize("ga,save_after_microbatches", [(1, 2), (3, 6), (3, 7)])
+def test_resume_continues_bit_identically(fixed_seed, mode, ga, save_after_microbatches):
+    """Four steps in one go against: stop after some micro-batches (at a step
+    boundary, or one micro-batch into an accumulation window), save, build a new
+    model and optimizer, load both, and finish.  Parameters and every state
+    tensor end up identical."""
+    import copy
+
+    from offload_adam_amd import OffloadAdam
+
+    steps = 4
+    data = batches(steps * ga)
+    kw = dict(mode=mode, lr=1e-2, weight_decay=0.01, inplace_param_threshold=5000,
+              max_grad_norm=None)
+
+    def build(seed):
+        model = make_model(seed)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            return model, OffloadAdam(model, **kw)
+
+    def run(model, opt, first, last):
+        for i in range(first, last):
+            opt.ready_for_optimizer_step = i % ga == ga - 1
+            loss_of(model, data[i]).backward()
+            if i % ga == ga - 1:
+                opt.step()
+                opt.zero_grad()
+        torch.cuda.synchronize()
+
+    ref_model, ref_opt = build(0)
+    run(ref_model, ref_opt, 0, steps * ga)
+
+    model, opt = build(0)
+    run(model, opt, 0, save_after_microbatches)
+    saved_opt = copy.deepcopy(opt.state_dict())
+    saved_model = copy.deepcopy(model.state_dict())
+    del model, opt
+
+    model2, opt2 = build(123)  # different initial weights: everything must come from the files
+    model2.load_state_dict(saved_model)
+    with pytest.raises(NotImplementedError):
+        opt2.load_state_dict(saved_opt)
+    opt2.load_offloaded_state_dict(saved_opt)
+    for st in opt2.state.values():  # still this optimizer's own kind of buffers
+        if "host_grad_valid" in st:
+            assert st["exp_avg"].is_pinned() and st["grad"].is_pinned()
+    run(model2, opt2, save_after_microbatches, steps * ga)
+
+    assert_same_params(ref_model, model2)
+    for pr, p2 in zip(ref_model.parameters(), model2.parameters()):
+        a, b = ref_opt.state[pr], opt2.state[p2]
+        assert set(a) == set(b)
+        for k in a:
+            if isinstance(a[k], torch.Tensor):
+                assert torch.equal(a[k].cpu(), b[k].cpu()), k
+            else:
+                assert a[k] == b[k], k
+
+
+def test_resume_rejects_a_state_that_does_not_fit(fixed_seed):
+    import copy
+
+    _, opt31 = run_offload_adam("fp31_master", 1, 1)
+    _, opt32 = run_offload_adam("fp32_master", 1, 1)
+    before = {k: v.clone() for k, v in next(iter(opt32.state.values())).items()
+              if isinstance(v, torch.Tensor)}
+    with pytest.raises(ValueError):
+        opt32.load_offloaded_state_dict(opt31.state_dict())
+    sd = copy.deepcopy(opt32.state_dict())
+    first = sd["state"][0]
+    first["exp_avg"] = first["exp_avg"][:1]
+    with pytest.raises(ValueError):
+        opt32.load_offloaded_state_dict(sd)
+    sd = copy.deepcopy(opt32.state_dict())
+    sd["param_groups"][0]["params"] = sd["param_groups"][0]["params"][:-1]
+    with pytest.raises(ValueError):
+        opt32.load_offloaded_state_dict(sd)
+    after = next(iter(opt32.state.values()))
+    for k, v in before.items():
+        assert torch.equal(after[k], v), "a rejected load changes nothing"
+
+
 def test_transfer_streams_are_picked_by_measured_concurrency():
     """With more live streams than hardware queues, the optimizer still ends up
     with side streams whose copies run beside each other and beside kernels."""
