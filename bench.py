@@ -5,7 +5,7 @@
 
 A "step" is one pass of the fused AdamW kernel over every tensor of the
 workload, with all operands already resident in HBM.  The default workload is
-BASELINE config 1: stochastic_rounding mode over the Llama-style 1.1B
+benchmark config 1: stochastic_rounding mode over the Llama-style 1.1B
 parameter set (201 tensors, 1,100,048,384 elements, 14 algorithmic bytes per
 element).  Prints ONE JSON line.
 
@@ -61,15 +61,15 @@ def llama_shapes(hidden, inter, layers, q_heads, kv_heads, head_dim, vocab):
 
 
 WORKLOADS = {
-    # BASELINE config 1
+    # benchmark config 1
     "c1_sr_llama1b": dict(
         mode="stochastic_rounding",
         shapes=llama_shapes(2048, 5632, 22, 32, 4, 64, 32000),
         clip=False,
     ),
-    # BASELINE config 0 (one flat tensor)
+    # benchmark config 0 (one flat tensor)
     "c0_fp32_master_16m": dict(mode="fp32_master", shapes=[("flat", (16_777_216,))], clip=False),
-    # BASELINE config 2 kernel leg: fp31_master + fused clip on Llama-3-8B shapes
+    # benchmark config 2 kernel leg: fp31_master + fused clip on Llama-3-8B shapes
     "c2_fp31_clip_llama8b": dict(
         mode="fp31_master",
         shapes=llama_shapes(4096, 14336, 32, 32, 8, 128, 128256),
@@ -159,7 +159,7 @@ def cpu_baseline(mode, target_elems=256 * 1024 * 1024, iters=5):
 
 def offloaded_step_8b(timeout_s=420):
     """The second half of the metric: step time of a synthetic Llama-3-8B-shaped
-    training step through OffloadAdam (BASELINE config 4), measured by
+    training step through OffloadAdam (benchmark config 4), measured by
     bench_e2e.py in a child process.  PCIe-inclusive; never part of ``value``."""
     import subprocess
 

@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """End-to-end synthetic training step with OffloadAdam on one MI355X
-(BASELINE config 4) and the host-link measurements that go with it.
+(benchmark config 4) and the host-link measurements that go with it.
 
     python bench_e2e.py [--model llama8b|llama1b|tiny] [--steps K] [--warmup W]
                         [--grad-accum 4] [--seq 4096] [--mode stochastic_rounding]
@@ -31,10 +31,10 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 MODELS = {
-    # BASELINE config 4 / config 2 shapes
+    # benchmark config 4 / config 2 shapes
     "llama8b": dict(hidden=4096, inter=14336, layers=32, q_heads=32, kv_heads=8, head_dim=128,
                     vocab=128256),
-    # BASELINE config 1 shapes
+    # benchmark config 1 shapes
     "llama1b": dict(hidden=2048, inter=5632, layers=22, q_heads=32, kv_heads=4, head_dim=64,
                     vocab=32000),
     "tiny": dict(hidden=256, inter=688, layers=2, q_heads=4, kv_heads=2, head_dim=64, vocab=1024),

@@ -216,7 +216,7 @@ def test_fp32_master_param_may_alias_grad(oracle):
 
 
 def test_config0_full_size(oracle):
-    """BASELINE config 0: one flat tensor of 16,777,216 elements, fp32_master,
+    """benchmark config 0: one flat tensor of 16,777,216 elements, fp32_master,
     lr=1e-4, betas=(0.9,0.999), eps=1e-8, wd=0.01 decoupled, step=10."""
     n = 16_777_216
     p, st = adam_inputs(n, seed=0, mode="fp32_master", device="cuda")
@@ -335,7 +335,7 @@ def test_argument_errors():
 
 
 def _llama_1b_shapes():
-    """The 201 parameter tensors of BASELINE config 1 (hidden 2048, MLP 5632, 22
+    """The 201 parameter tensors of benchmark config 1 (hidden 2048, MLP 5632, 22
     layers, 32 query / 4 key-value heads of 64, vocabulary 32000, untied)."""
     h, inter, layers, kv, vocab = 2048, 5632, 22, 4 * 64, 32000
     shapes = [(vocab, h)]
@@ -346,7 +346,7 @@ def _llama_1b_shapes():
 
 
 def test_config1_full_set(oracle):
-    """BASELINE config 1 at full size: 201 tensors, 1,100,048,384 elements,
+    """benchmark config 1 at full size: 201 tensors, 1,100,048,384 elements,
     stochastic rounding, one multi-tensor step (6 launches).
 
     * one tensor of every distinct size (82 M elements) is compared bit for bit

@@ -4,7 +4,7 @@ packed codes, the scales and the dequantised values.
 Shapes follow the reference's own parity tests (tests/test_int8.py:70-84 and
 the other three files): seeded ``randn * 0.05`` in bf16 / fp16, plus fp32
 masters, misaligned row counts, column counts off the 8-element fast path,
-strided and unaligned sources, and BASELINE config 3 (4096 x 14336 with 1 %
+strided and unaligned sources, and benchmark config 3 (4096 x 14336 with 1 %
 outliers x10).
 """
 
@@ -234,7 +234,7 @@ def test_nvfp4_e2m1_boundaries_match_bit_level_definition(oracle):
 
 
 def test_config3_weight(oracle):
-    """BASELINE config 3: 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
+    """benchmark config 3: 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
     x10; requantise from its fp32 master, every format, then dequantise."""
     from offload_adam_amd.qweight import _codec_ops as ops
 

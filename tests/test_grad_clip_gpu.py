@@ -112,7 +112,7 @@ def test_fused_clip_equals_separate_mul(mode):
 
 
 def test_config2_norm_and_clip_flow(oracle):
-    """BASELINE config 2 shape of the flow at reduced tensor sizes: grads scaled
+    """benchmark config 2 shape of the flow at reduced tensor sizes: grads scaled
     so the global norm is ~3 with max_grad_norm=1 (coef ~ 1/3)."""
     from offload_adam_amd.grad_clip import clip_coef_, grad_norm_
 
@@ -135,7 +135,7 @@ def test_config2_norm_and_clip_flow(oracle):
 
 
 def _llama_8b_shapes():
-    """The 291 parameter tensors of BASELINE config 2 / 4 (hidden 4096, MLP 14336,
+    """The 291 parameter tensors of benchmark config 2 / 4 (hidden 4096, MLP 14336,
     32 layers, 32 query / 8 key-value heads of 128, vocabulary 128256, untied)."""
     h, inter, layers, kv, vocab = 4096, 14336, 32, 8 * 128, 128256
     shapes = [(vocab, h)]
@@ -146,7 +146,7 @@ def _llama_8b_shapes():
 
 
 def test_config2_full_set(oracle):
-    """BASELINE config 2 at full size, kernel legs on GPU-resident buffers: 291
+    """benchmark config 2 at full size, kernel legs on GPU-resident buffers: 291
     tensors, 8,030,261,248 elements, fp31_master, gradients with a global norm of
     about 3 clipped to max_grad_norm = 1 inside the AdamW kernel.
 
