@@ -626,11 +626,13 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
     from offload_adam_amd import offload_adam as oa_mod
 
     log = []
-    real = {n: getattr(oa_mod.OffloadAdam, n) for n in ("_issue_h2d", "_issue_d2h", "_call_step_fn")}
+    real = {n: getattr(oa_mod.OffloadAdam, n)
+            for n in ("_issue_h2d_many", "_issue_d2h", "_call_step_fn")}
 
-    def h2d(self, p, keys):
-        log.append(("h2d", p, tuple(keys)))
-        return real["_issue_h2d"](self, p, keys)
+    def h2d(self, items):  # every fetch goes through the batched form
+        for p, keys in items:
+            log.append(("h2d", p, tuple(keys)))
+        return real["_issue_h2d_many"](self, items)
 
     def d2h(self, p, keys):
         log.append(("d2h", p, tuple(keys)))
@@ -640,7 +642,7 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
         log.append(("step", p, tuple(tensors)))
         return real["_call_step_fn"](self, p, group, tensors, clip_coef)
 
-    monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_h2d", h2d)
+    monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_h2d_many", h2d)
     monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_d2h", d2h)
     monkeypatch.setattr(oa_mod.OffloadAdam, "_call_step_fn", step)
     steps, ga = 3, 3
