@@ -549,6 +549,61 @@ def test_resume_rejects_a_state_that_does_not_fit(fixed_seed):
         assert torch.equal(after[k], v), "a rejected load changes nothing"
 
 
+class BranchyNet(TinyNet):
+    """TinyNet whose middle block is skipped for odd ``route`` and whose head is
+    one of two: some parameters get no gradient in some passes."""
+
+    def __init__(self):
+        super().__init__()
+        self.head2 = nn.Linear(96, 50, bias=False)
+
+    def forward(self, ids, route=0):
+        x = self.emb(ids)
+        for i, b in enumerate(self.blocks):
+            if i == 1 and route % 2:
+                continue
+            x = x + b["down"](F.gelu(b["up"](b["norm"](x))))
+        return (self.head2 if route % 3 == 2 else self.head)(x)
+
+
+@pytest.mark.parametrize("mode", ["fp31_master", "stochastic_rounding"])
+@pytest.mark.parametrize("kw", [dict(), dict(prefetch_bytes=0), dict(offload_grads=False)])
+def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
+    """The order of gradient hooks is learned, and prefetch runs along it; passes
+    that skip modules (their hooks never fire, their prefetched states are not
+    consumed) must neither stall nor change a result.  Every step uses one route
+    for all its micro-batches, so the optimizer without offloading sees the same
+    set of gradients."""
+    from offload_adam_amd import Adam, OffloadAdam
+
+    steps, ga = 7, 2
+    data = batches(steps * ga)
+
+    def train(make_opt, offloaded):
+        torch.manual_seed(0)
+        model = BranchyNet().to(device="cuda", dtype=BF16)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            opt = make_opt(model)
+        for s in range(steps):
+            for mb in range(ga):
+                if offloaded:
+                    opt.ready_for_optimizer_step = mb == ga - 1
+                out = model(data[s * ga + mb], route=s)
+                F.cross_entropy(out.float().reshape(-1, 50), data[s * ga + mb].reshape(-1)).backward()
+            opt.step()
+            opt.zero_grad(*([] if offloaded else [True]))
+        torch.cuda.synchronize()
+        return model, opt
+
+    ref, _ = train(lambda m: Adam(m.parameters(), mode=mode, lr=1e-2, weight_decay=0.01), False)
+    got, opt = train(lambda m: OffloadAdam(m, mode=mode, lr=1e-2, weight_decay=0.01,
+                                           inplace_param_threshold=5000, **kw), True)
+    assert_same_params(ref, got)
+    used = [opt.state[p]["step"] for p in got.parameters()]
+    assert min(used) < steps and max(used) == steps  # some parameters did skip steps
+
+
 def test_transfer_streams_are_picked_by_measured_concurrency():
     """With more live streams than hardware queues, the optimizer still ends up
     with side streams whose copies run beside each other and beside kernels."""
