@@ -173,10 +173,23 @@ def measure_link(nbytes=1 << 30, reps=5):
         return nbytes * reps / (time.perf_counter() - t0) / 1e9
 
     run(True, True)  # warm-up
+
+    def best(*what):
+        # The best of up to five, with pauses: a process started right after one
+        # that held tens of GiB of pinned memory measures D2H at 30 GB/s instead
+        # of 57 for its first seconds (the driver is still releasing those pages).
+        rates = []
+        for _ in range(5):
+            rates.append(run(*what))
+            if rates[-1] > 45.0:
+                break
+            time.sleep(1.0)
+        return round(max(rates), 2)
+
     return {
-        "h2d_GBps": round(run(True, False), 2),
-        "d2h_GBps": round(run(False, True), 2),
-        "bidir_each_GBps": round(run(True, True), 2),
+        "h2d_GBps": best(True, False),
+        "d2h_GBps": best(False, True),
+        "bidir_each_GBps": best(True, True),
         "dma_h2d_plus_kernel_d2h_each_GBps": {wg: round(run_mixed(wg), 2) for wg in (4, 8, 16)},
     }
 
@@ -190,11 +203,14 @@ def link_bytes_per_step(opt, grad_accum):
                   for k, d in opt.offload_config.items() if k != "grad")
     if not opt.offload_grads:
         h2d = d2h = n * state_b
-    elif opt._step_in_backward:
-        h2d = n * (2 * (grad_accum - 1) + state_b)
+        return h2d, d2h
+    # gradients kept on the GPU after their write-back are never fetched again
+    fetched = sum(p.numel() for p in opt._offload_params if p not in opt._grad_cached)
+    if opt._step_in_backward:
+        h2d = n * state_b + fetched * 2 * (grad_accum - 1)
         d2h = n * (2 * (grad_accum - 1) + state_b)
     else:
-        h2d = n * (2 * (grad_accum - 1) + 2 + state_b)
+        h2d = n * state_b + fetched * 2 * grad_accum
         d2h = n * (2 * grad_accum + state_b)
     return h2d, d2h
 
@@ -331,12 +347,15 @@ def run(args):
         opt = OffloadAdam(model, lr=1e-5, mode=args.mode, max_grad_norm=args.max_grad_norm,
                           inplace_param_threshold=1024 * 1024, prefetch_policy="eager",
                           decoupled_weight_decay=True, offload_grads=not args.grads_on_device,
-                          prefetch_bytes=int(args.prefetch_gib * 2**30) if args.prefetch_gib else None)
+                          prefetch_bytes=int(args.prefetch_gib * 2**30) if args.prefetch_gib else None,
+                          grad_cache_bytes=(None if args.grad_cache_gib is None
+                                            else int(args.grad_cache_gib * 2**30)))
     torch.cuda.synchronize()
     out["optimizer_init_s"] = round(time.perf_counter() - t0, 2)
     out["offloaded_params"] = len(opt._offload_params)
     out["inplace_params"] = len(opt._inplace_params)
     out["prefetch_GiB"] = round(opt._PREFETCH_BYTES / 1024**3, 2)
+    out["grad_cache_GiB"] = round(sum(p.numel() for p in opt._grad_cached) * 2 / 1024**3, 2)
     out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
 
     timeline = None
@@ -361,8 +380,11 @@ def run(args):
     out["d2h_GB_per_step"] = round(d2h / 1e9, 2)
     out["h2d_GBps_over_step"] = round(h2d / step_s / 1e9, 2)
     out["d2h_GBps_over_step"] = round(d2h / step_s / 1e9, 2)
-    peak = out["link_peak"]["bidir_each_GBps"]
-    out["link_floor_s"] = round(max(h2d, d2h) / 1e9 / peak, 4)
+    # no schedule can beat: each direction at its solo rate, both together at twice
+    # the rate each reaches while the other is busy
+    peaks = out["link_peak"]
+    out["link_floor_s"] = round(max(h2d / 1e9 / peaks["h2d_GBps"], d2h / 1e9 / peaks["d2h_GBps"],
+                                    (h2d + d2h) / 1e9 / (2 * peaks["bidir_each_GBps"])), 4)
     out["transfer_streams"] = opt.transfer_stream_report
     st = _copy_engines.status()
     out["copy_engines"] = {k: st.get(k) for k in ("loaded", "active", "h2d_engine", "d2h_engine",
@@ -415,6 +437,10 @@ def main():
     ap.add_argument("--qat", default=None, choices=["int8", "int4", "nf4", "nvfp4"],
                     help="quantise every decoder Linear weight (lm_head excluded) and train "
                          "against fp32 masters: implies --mode fp32_master")
+    ap.add_argument("--grad-cache-gib", type=float, default=None,
+                    help="OffloadAdam(grad_cache_bytes=...): HBM for gradients kept on the GPU "
+                         "after their write-back (default: the optimizer's; 0 = fetch every time "
+                         "like the reference)")
     ap.add_argument("--grads-on-device", action="store_true",
                     help="OffloadAdam(offload_grads=False): the gradient sum stays in HBM")
     ap.add_argument("--copy-timeline", action="store_true",

@@ -39,6 +39,11 @@ void oa_copy_engines_config(unsigned* h2d_mask, unsigned* d2h_mask);
 void oa_copy_engines_stats(unsigned long long* h2d_copies, unsigned long long* d2h_copies,
                            unsigned long long* rejected);
 
+/* Host<->device copies that reached the runtime through the call that names no
+ * engine (hsa_amd_memory_async_copy) and were sent to the fixed engines as well;
+ * they are included in the per-direction counts above. */
+unsigned long long oa_copy_engines_unpinned_calls(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -53,7 +53,7 @@ def install():
 def status():
     """What the tools library reports once the GPU runtime is up:
     ``{"install", "loaded", "active", "h2d_engine", "d2h_engine", "h2d_copies",
-    "d2h_copies", "rejected"}``.  ``loaded`` is False when the runtime started
+    "d2h_copies", "rejected", "unpinned_calls"}``.  ``loaded`` is False when the runtime started
     before :func:`install` ran (or the library is missing)."""
     out = {"install": _install_result, "loaded": False, "active": False}
     if not LIB_PATH.exists():
@@ -71,4 +71,6 @@ def status():
     a, b, c = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
     lib.oa_copy_engines_stats(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))
     out["h2d_copies"], out["d2h_copies"], out["rejected"] = a.value, b.value, c.value
+    lib.oa_copy_engines_unpinned_calls.restype = ctypes.c_ulonglong
+    out["unpinned_calls"] = lib.oa_copy_engines_unpinned_calls()
     return out

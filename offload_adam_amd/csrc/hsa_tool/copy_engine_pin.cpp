@@ -43,13 +43,14 @@
 namespace {
 
 decltype(hsa_amd_memory_async_copy_on_engine)* real_copy_on_engine = nullptr;
+decltype(hsa_amd_memory_async_copy)* real_copy = nullptr;
 decltype(hsa_agent_get_info)* real_agent_get_info = nullptr;
 
 std::atomic<int> loaded{0};
 std::atomic<int> active{0};
 unsigned h2d_engine = 0x1;
 unsigned d2h_engine = 0x2;
-std::atomic<unsigned long long> n_h2d{0}, n_d2h{0}, n_rejected{0};
+std::atomic<unsigned long long> n_h2d{0}, n_d2h{0}, n_rejected{0}, n_unpinned{0};
 std::atomic<int> rejected_in_a_row{0};
 constexpr int kMaxRejectedInARow = 8;
 
@@ -89,6 +90,35 @@ hsa_status_t copy_on_fixed_engine(void* dst, hsa_agent_t dst_agent, const void* 
                              completion_signal, engine_id, force_copy_on_sdma);
 }
 
+// The runtime's other copy call names no engine and lets ROCr choose one (HIP
+// falls back to it when the engine status query offers nothing).  Host<->device
+// copies that arrive here are sent to the same fixed engines; a rejected rewrite
+// falls through to the call as it was made.
+hsa_status_t copy_without_engine(void* dst, hsa_agent_t dst_agent, const void* src,
+                                 hsa_agent_t src_agent, size_t size, uint32_t num_dep_signals,
+                                 const hsa_signal_t* dep_signals,
+                                 hsa_signal_t completion_signal) {
+  if (active.load(std::memory_order_relaxed)) {
+    const bool src_cpu = is_cpu(src_agent), dst_cpu = is_cpu(dst_agent);
+    unsigned want = 0;
+    if (src_cpu && !dst_cpu) want = h2d_engine;
+    else if (!src_cpu && dst_cpu) want = d2h_engine;
+    if (want != 0) {
+      n_unpinned.fetch_add(1, std::memory_order_relaxed);
+      hsa_status_t st = real_copy_on_engine(dst, dst_agent, src, src_agent, size, num_dep_signals,
+                                            dep_signals, completion_signal,
+                                            static_cast<hsa_amd_sdma_engine_id_t>(want), false);
+      if (st == HSA_STATUS_SUCCESS) {
+        (src_cpu ? n_h2d : n_d2h).fetch_add(1, std::memory_order_relaxed);
+        return st;
+      }
+      n_rejected.fetch_add(1, std::memory_order_relaxed);
+    }
+  }
+  return real_copy(dst, dst_agent, src, src_agent, size, num_dep_signals, dep_signals,
+                   completion_signal);
+}
+
 // "0x1,0x2" -> masks; anything malformed keeps the defaults.  Returns false for "off".
 bool read_config() {
   const char* s = getenv("OFFLOAD_ADAM_COPY_ENGINES");
@@ -115,6 +145,10 @@ extern "C" bool OnLoad(HsaApiTable* table, uint64_t /*runtime_version*/,
   real_agent_get_info = table->core_->hsa_agent_get_info_fn;
   real_copy_on_engine = table->amd_ext_->hsa_amd_memory_async_copy_on_engine_fn;
   table->amd_ext_->hsa_amd_memory_async_copy_on_engine_fn = copy_on_fixed_engine;
+  if (table->amd_ext_->hsa_amd_memory_async_copy_fn) {
+    real_copy = table->amd_ext_->hsa_amd_memory_async_copy_fn;
+    table->amd_ext_->hsa_amd_memory_async_copy_fn = copy_without_engine;
+  }
   active.store(rewrite ? 1 : 0);
   loaded.store(1);
   return true;
@@ -130,6 +164,8 @@ extern "C" void oa_copy_engines_config(unsigned* h2d_mask, unsigned* d2h_mask) {
   if (h2d_mask) *h2d_mask = h2d_engine;
   if (d2h_mask) *d2h_mask = d2h_engine;
 }
+
+extern "C" unsigned long long oa_copy_engines_unpinned_calls(void) { return n_unpinned.load(); }
 
 extern "C" void oa_copy_engines_stats(unsigned long long* h2d_copies, unsigned long long* d2h_copies,
                                       unsigned long long* rejected) {

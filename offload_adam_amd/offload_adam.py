@@ -221,6 +221,15 @@ class OffloadAdam(Optimizer):
             with ``grad_accum`` micro-batches the link traffic per step drops
             from ``2*(grad_accum-1)+4`` to ``4`` bytes per element each way in
             ``stochastic_rounding`` mode.  Results are bit-identical.
+        grad_cache_bytes (int, keyword-only): with ``offload_grads=True``, HBM
+            that may keep the device copy of accumulated gradients alive after
+            they have been written back to the host.  The write-back happens as
+            in the reference (``state[p]['grad']`` on the host is always
+            current); what is saved is fetching the same bytes again for the next
+            micro-batch, or for ``step()`` on the clipping path.  Parameters are
+            admitted in optimizer order until the budget is used.  Default: a
+            tenth of the HBM that is free when the optimizer is built; ``0``
+            fetches every time, like the reference.  Results are bit-identical.
     """
 
     supported_modes = {
@@ -253,6 +262,7 @@ class OffloadAdam(Optimizer):
         *,
         offload_grads=True,
         prefetch_bytes=None,
+        grad_cache_bytes=None,
     ):
         if prefetch_policy not in ("eager", "lazy"):
             raise ValueError(f"prefetch_policy must be 'eager' or 'lazy' (got {prefetch_policy!r})")
@@ -269,6 +279,8 @@ class OffloadAdam(Optimizer):
         self._prefetch_bytes_arg = prefetch_bytes
         if prefetch_bytes is not None:
             self._PREFETCH_BYTES = int(prefetch_bytes)
+        if grad_cache_bytes is not None and grad_cache_bytes < 0:
+            raise ValueError("grad_cache_bytes must be >= 0")
         # what lives in pinned host memory between steps
         self._host_config = {
             k: d for k, d in self.offload_config.items() if k != "grad" or self.offload_grads
@@ -324,6 +336,20 @@ class OffloadAdam(Optimizer):
             if dev0.type == "cuda":
                 free, _ = torch.cuda.mem_get_info(dev0)
                 self._PREFETCH_BYTES = max(2 << 30, free // 10)
+
+        # parameters whose accumulated gradient stays on the GPU after its write-back
+        self._grad_cached = set()
+        if self.offload_grads and self._offload_params:
+            budget = grad_cache_bytes
+            if budget is None:
+                dev0 = self._offload_params[0].device
+                budget = torch.cuda.mem_get_info(dev0)[0] // 10 if dev0.type == "cuda" else 0
+            for p in self._offload_params:
+                nbytes = p.numel() * 2
+                if nbytes > budget:
+                    break
+                budget -= nbytes
+                self._grad_cached.add(p)
 
         self.device_states = {}
         self.h2d_events = {}
@@ -549,7 +575,8 @@ class OffloadAdam(Optimizer):
             else:
                 _copy_async(self._host_view(p, key), buf, _lib.OA_COPY_D2H, self.d2h_stream)
             buf.record_stream(self.d2h_stream)
-            dev[key] = None
+            if key != "grad" or p not in self._grad_cached:
+                dev[key] = None
         self.d2h_events[p] = self.d2h_stream.record_event()
 
     def _ensure_on_device(self, p, keys):
@@ -573,6 +600,10 @@ class OffloadAdam(Optimizer):
             else:
                 dev["grad"].add_(p.grad)
         elif state["host_grad_valid"]:
+            if dev.get("grad") is not None and p in self.d2h_events:
+                # the device copy was kept (grad_cache_bytes): its write-back to the
+                # host must have read it before the sum below overwrites it
+                self._compute_stream().wait_event(self.d2h_events[p])
             self._ensure_on_device(p, ["grad"])
             dev["grad"].add_(p.grad)
         else:
@@ -730,11 +761,13 @@ class OffloadAdam(Optimizer):
         first ``prefetch_bytes`` of them (in the order ``step()`` walks the
         parameters) cross the link under the last backward pass instead of
         inside ``step()``.  Not when this pass has to fetch accumulated gradients
-        from the host: the host->device direction is then busy for the whole pass
+        from the host (none of those kept on the GPU by ``grad_cache_bytes``
+        count): the host->device direction is then busy for the whole pass
         and staged states would only queue ahead of the gradients backward waits
         for (measured: 2.86 s instead of 2.71 s per 8B step)."""
         if self.offload_grads and any(
-            self.state[p]["host_grad_valid"] for p in self._offload_params
+            self.state[p]["host_grad_valid"] and self.device_states[p].get("grad") is None
+            for p in self._offload_params
         ):
             return
         budget = self._PREFETCH_BYTES

@@ -26,7 +26,7 @@ def test_library_exports_header_symbols_and_tool_entry_points():
     lib = ctypes.CDLL(str(_copy_engines.LIB_PATH))
     names = declared()
     assert names == ["oa_copy_engines_active", "oa_copy_engines_config", "oa_copy_engines_loaded",
-                     "oa_copy_engines_stats"]
+                     "oa_copy_engines_stats", "oa_copy_engines_unpinned_calls"]
     for name in names + ["OnLoad", "OnUnload"]:
         assert hasattr(lib, name), name
 

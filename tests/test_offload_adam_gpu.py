@@ -604,6 +604,54 @@ def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
     assert min(used) < steps and max(used) == steps  # some parameters did skip steps
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("cache", [0, 40_000, None])
+@pytest.mark.parametrize("clip", [None, 0.05])
+def test_gradient_cache_does_not_change_results(fixed_seed, mode, cache, clip):
+    """grad_cache_bytes = 0 (every accumulated gradient is fetched back, as in the
+    reference), a budget that admits only some parameters, and the default: same
+    bits as the optimizer without offloading, on the hook path and the clip path;
+    the host copy of the gradient sum is current in every case."""
+    if clip is None:
+        ref_model, _ = run_reference_adam(mode, steps=3, ga=3)
+    else:
+        ref_model, _ = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip,
+                                        grad_cache_bytes=0)
+    model, opt = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip, grad_cache_bytes=cache)
+    assert_same_params(ref_model, model)
+    n_cached = len(opt._grad_cached)
+    if cache == 0:
+        assert n_cached == 0
+    elif cache is None:
+        assert n_cached == len(opt._offload_params)
+    else:
+        assert 0 < n_cached < len(opt._offload_params)
+
+
+def test_cached_gradient_is_also_current_on_the_host(fixed_seed):
+    """One micro-batch into a window: the pinned ``state['grad']`` holds the same
+    sum whether or not the device copy was kept."""
+    from offload_adam_amd import OffloadAdam
+
+    sums = []
+    for cache in (0, None):
+        model = make_model(0)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, inplace_param_threshold=5000,
+                              grad_cache_bytes=cache)
+        data = batches(2)
+        for mb in range(2):
+            opt.ready_for_optimizer_step = False
+            loss_of(model, data[mb]).backward()
+        torch.cuda.synchronize()
+        sums.append([opt.state[p]["grad"].clone() for p in opt._offload_params])
+        kept = [opt.device_states[p].get("grad") is not None for p in opt._offload_params]
+        assert all(kept) if cache is None else not any(kept)
+    for a, b in zip(*sums):
+        assert torch.equal(a, b) and a.abs().sum() > 0
+
+
 def test_transfer_streams_are_picked_by_measured_concurrency():
     """With more live streams than hardware queues, the optimizer still ends up
     with side streams whose copies run beside each other and beside kernels."""
@@ -671,7 +719,9 @@ def test_prefetch_budget_does_not_change_results(fixed_seed, prefetch_bytes):
 
 
 @pytest.mark.parametrize("kw", [dict(), dict(max_grad_norm=0.05), dict(offload_grads=False),
-                                dict(prefetch_bytes=0)])
+                                dict(prefetch_bytes=0), dict(grad_cache_bytes=0),
+                                dict(grad_cache_bytes=0, max_grad_norm=0.05),
+                                dict(grad_cache_bytes=40_000)])
 def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monkeypatch, kw):
     """Log every H2D / kernel / D2H the optimizer issues and check, per parameter
     and state key: a key is on the device (H2D issued, not yet written back) when
@@ -711,12 +761,14 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
             continue
         if op == "h2d":
             for k in keys:
-                assert not on_device.get((p, k)), f"{k} fetched twice without a write-back"
+                assert not on_device.get((p, k)), f"{k} fetched while a copy is on the device"
                 on_device[(p, k)] = True
         elif op == "d2h":
             for k in keys:
-                if k != "grad" or opt.offload_grads:
-                    on_device[(p, k)] = False
+                if k == "grad" and not opt.offload_grads:
+                    continue
+                # a cached gradient is written back and stays on the GPU as well
+                on_device[(p, k)] = k == "grad" and p in opt._grad_cached
         else:
             stepped[p] += 1
             for k in opt._non_grad_keys:
