@@ -242,6 +242,14 @@ class OffloadAdam(Optimizer):
 
     _DEFAULT_INPLACE_PARAM_THRESHOLD = 1024 * 1024
     _CLIP_PREFETCH_DEPTH = 2  # parameters whose H2D runs ahead of the step loop
+    # Hook path: parameters whose gradient is complete are stepped in groups - one
+    # multi-tensor launch, one fence and one event for the write-back of the whole
+    # group - because the host cost of a hook (about 85 us per parameter when each
+    # is stepped alone, mostly stream waits and launches) is what a step of a
+    # 1B-parameter model is bound by.  A group closes at this many parameters or
+    # bytes of gradient, whichever comes first, and when the backward pass ends.
+    _STEP_GROUP_PARAMS = 8
+    _STEP_GROUP_BYTES = 256 << 20
     _PREFETCH_MIN_PARAMS = 2  # hook path: H2D window ahead of the gradient hooks ...
     _PREFETCH_BYTES = 8 << 30  # ... and in bytes of device staging (re-derived per instance)
 
@@ -351,6 +359,10 @@ class OffloadAdam(Optimizer):
                 budget -= nbytes
                 self._grad_cached.add(p)
 
+        self._pending_steps = []      # offloaded parameters waiting for their group's launch
+        self._pending_inplace = []    # GPU-resident ones
+        self._pending_step_bytes = 0
+        self._flush_callback_queued = False
         self.device_states = {}
         self.h2d_events = {}
         self.d2h_events = {}
@@ -579,6 +591,25 @@ class OffloadAdam(Optimizer):
                 dev[key] = None
         self.d2h_events[p] = self.d2h_stream.record_event()
 
+    def _issue_d2h_many(self, items):
+        """Write-back of ``keys`` of every ``(p, keys)`` behind one fence, with one
+        event for the group (a later fetch of any of them waits for all)."""
+        if not items:
+            return
+        d2h = self.d2h_stream
+        d2h.wait_stream(self._compute_stream())
+        for p, keys in items:
+            dev = self.device_states[p]
+            for key in keys:
+                buf = dev[key]
+                _copy_async(self._host_view(p, key), buf, _lib.OA_COPY_D2H, d2h)
+                buf.record_stream(d2h)
+                if key != "grad" or p not in self._grad_cached:
+                    dev[key] = None
+        event = d2h.record_event()
+        for p, _ in items:
+            self.d2h_events[p] = event
+
     def _ensure_on_device(self, p, keys):
         dev = self.device_states[p]
         missing = [k for k in keys if dev.get(k) is None]
@@ -679,6 +710,89 @@ class OffloadAdam(Optimizer):
         )
         torch._foreach_zero_([t["grad"] for t in tensors])
 
+    def _queue_step(self, p, inplace=False):
+        """Hook path: ``p``'s gradient is complete; step it with its group."""
+        if inplace:
+            self._pending_inplace.append(p)
+        else:
+            self._pending_steps.append(p)
+        self._pending_step_bytes += p.numel() * 2
+        if not self._flush_callback_queued:
+            # runs when this backward pass has executed its last node: no group is
+            # ever left waiting for a hook that does not come
+            try:
+                torch.autograd.Variable._execution_engine.queue_callback(self._flush_steps)
+                self._flush_callback_queued = True
+            except RuntimeError:  # called outside a backward pass: nothing to wait for
+                self._flush_steps()
+                return
+        if (len(self._pending_steps) + len(self._pending_inplace) >= self._STEP_GROUP_PARAMS
+                or self._pending_step_bytes >= self._STEP_GROUP_BYTES):
+            self._flush_steps(final=False)
+
+    @torch.no_grad()
+    def _flush_steps(self, final=True):
+        """Step every queued parameter: fetch what is missing (one fence), one
+        multi-tensor launch per param group, one fenced write-back."""
+        if final:
+            self._flush_callback_queued = False
+        offloaded, inplace = self._pending_steps, self._pending_inplace
+        if not offloaded and not inplace:
+            return
+        self._pending_steps, self._pending_inplace, self._pending_step_bytes = [], [], 0
+        if inplace:
+            by_group = {}
+            for p in inplace:
+                by_group.setdefault(id(self._param2group[p]), []).append(p)
+            for members in by_group.values():
+                self._step_inplace_batch(members, self._param2group[members[0]])
+        if not offloaded:
+            return
+        if _trace.ENABLED:
+            with _trace.range(f"oa.steps x{len(offloaded)}"):
+                self._step_offload_group(offloaded)
+        else:
+            self._step_offload_group(offloaded)
+
+    def _step_offload_group(self, params):
+        missing = []
+        for p in params:
+            dev = self.device_states[p]
+            keys = [k for k in self.offload_state_keys if dev.get(k) is None]
+            if keys:
+                missing.append((p, keys))
+        self._issue_h2d_many(missing)
+        compute = self._compute_stream()
+        waited = set()
+        for p in params:
+            event = self.h2d_events.get(p)
+            if event is not None and id(event) not in waited:
+                compute.wait_event(event)
+                waited.add(id(event))
+        by_group = {}
+        for p in params:
+            state = self.state[p]
+            state["step"] += 1
+            group = self._param2group[p]
+            dev = self.device_states[p]
+            if p in self._quant_params or not (p.data.is_contiguous() and p.dtype == _BF16):
+                self._call_step_fn(p, group, dev)  # its own launch (re-encodes the payload)
+            else:
+                by_group.setdefault(id(group), (group, [], [], []))
+                _, ps, tensors, steps = by_group[id(group)]
+                ps.append(p.data)
+                tensors.append(dev)
+                steps.append(state["step"])
+        for group, ps, tensors, steps in by_group.values():
+            beta1, beta2 = group["betas"]
+            adam_step_multi(self.mode, ps, tensors, group["lr"], group["weight_decay"], beta1,
+                            beta2, group["eps"], steps,
+                            decoupled_weight_decay=self.decoupled_weight_decay)
+        self._issue_d2h_many([(p, self._non_grad_keys) for p in params])
+        for p in params:
+            self.device_states[p]["grad"] = None
+            self.state[p]["host_grad_valid"] = False
+
     def _record_grad_norm(self, p, grad):
         grad_clip.grad_norm_(grad.reshape(-1), self.state[p]["grad_norm"])
 
@@ -746,6 +860,8 @@ class OffloadAdam(Optimizer):
         copies, so they run under that forward pass instead of waiting for the
         first backward hook."""
         self._ready_for_optimizer_step = bool(value)
+        if getattr(self, "_pending_steps", None) or getattr(self, "_pending_inplace", None):
+            self._flush_steps()
         if not self._ready_for_optimizer_step or not hasattr(self, "_bw_order"):
             return
         if self._step_in_backward:
@@ -830,10 +946,9 @@ class OffloadAdam(Optimizer):
         if self.max_grad_norm is not None and last:
             self._record_grad_norm(p, self.device_states[p]["grad"])
         if self._step_in_backward and last:
-            state["step"] += 1
-            self._step_offload(p, self._param2group[p])
-            state["host_grad_valid"] = False
+            self._queue_step(p)
             if self._bw_order_known and pos == len(self._bw_order) - 1:
+                self._flush_steps(final=False)
                 # The step is complete.  The host->device direction is idle until
                 # the next accumulation pass needs gradients back (never, with
                 # offload_grads=False): stage the states the next step touches
@@ -853,8 +968,7 @@ class OffloadAdam(Optimizer):
         if self.max_grad_norm is not None and last:
             self._record_grad_norm(p, state["grad"])
         if self._step_in_backward and last:
-            state["step"] += 1
-            self._step_inplace(p, self._param2group[p])
+            self._queue_step(p, inplace=True)
 
     # ------------------------------------------------------------- public API
 
@@ -868,6 +982,7 @@ class OffloadAdam(Optimizer):
             )
         self._bw_cursor = -1  # the next backward pass starts a new prefetch window
         if self._step_in_backward:
+            self._flush_steps()  # normally empty: the end of backward has flushed
             return
 
         clip_coef = None
@@ -906,6 +1021,12 @@ class OffloadAdam(Optimizer):
     def zero_grad(self, set_to_none=False):
         """No-op: gradients are consumed by the hooks."""
         return
+
+    def state_dict(self):
+        """``Optimizer.state_dict()``; parameters still waiting for their group's
+        launch are stepped first."""
+        self._flush_steps()
+        return super().state_dict()
 
     @torch.no_grad()
     def load_master_state_dict(self, state_dict, model, strict=False):
@@ -973,6 +1094,7 @@ class OffloadAdam(Optimizer):
         unless the optimizer was built with ``offload_grads=False``, whose running
         sums never reach the state dict.
         """
+        self._flush_steps()
         saved_groups = state_dict["param_groups"]
         saved_state = state_dict["state"]
         if len(saved_groups) != len(self.param_groups):

@@ -732,7 +732,8 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
 
     log = []
     real = {n: getattr(oa_mod.OffloadAdam, n)
-            for n in ("_issue_h2d_many", "_issue_d2h", "_call_step_fn")}
+            for n in ("_issue_h2d_many", "_issue_d2h", "_issue_d2h_many", "_call_step_fn")}
+    real_multi = oa_mod.adam_step_multi
 
     def h2d(self, items):  # every fetch goes through the batched form
         for p, keys in items:
@@ -743,13 +744,34 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
         log.append(("d2h", p, tuple(keys)))
         return real["_issue_d2h"](self, p, keys)
 
+    def d2h_many(self, items):
+        for p, keys in items:
+            log.append(("d2h", p, tuple(keys)))
+        return real["_issue_d2h_many"](self, items)
+
     def step(self, p, group, tensors, clip_coef=None):
         log.append(("step", p, tuple(tensors)))
         return real["_call_step_fn"](self, p, group, tensors, clip_coef)
 
+    by_address = {}
+
+    def multi(mode, params, states, *args, **kwargs):  # the grouped launch of the hook path
+        for data, tensors in zip(params, states):
+            log.append(("step", by_address[data.data_ptr()], tuple(tensors)))
+        return real_multi(mode, params, states, *args, **kwargs)
+
     monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_h2d_many", h2d)
     monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_d2h", d2h)
+    monkeypatch.setattr(oa_mod.OffloadAdam, "_issue_d2h_many", d2h_many)
     monkeypatch.setattr(oa_mod.OffloadAdam, "_call_step_fn", step)
+    monkeypatch.setattr(oa_mod, "adam_step_multi", multi)
+    real_init = oa_mod.OffloadAdam.__init__
+
+    def init(self, model, *a, **k):
+        by_address.update({q.data_ptr(): q for q in model.parameters()})
+        return real_init(self, model, *a, **k)
+
+    monkeypatch.setattr(oa_mod.OffloadAdam, "__init__", init)
     steps, ga = 3, 3
     model, opt = run_offload_adam("fp31_master", steps=steps, ga=ga, **kw)
     offloaded = set(opt._offload_params)
