@@ -652,6 +652,67 @@ def test_cached_gradient_is_also_current_on_the_host(fixed_seed):
         assert torch.equal(a, b) and a.abs().sum() > 0
 
 
+@pytest.mark.parametrize("group_params,group_bytes", [(1, 1 << 30), (3, 1 << 30), (100, 1 << 30),
+                                                      (100, 40_000)])
+def test_step_groups_of_any_size_give_the_same_result(fixed_seed, monkeypatch, group_params,
+                                                      group_bytes):
+    from offload_adam_amd import offload_adam as oa_mod
+
+    monkeypatch.setattr(oa_mod.OffloadAdam, "_STEP_GROUP_PARAMS", group_params)
+    monkeypatch.setattr(oa_mod.OffloadAdam, "_STEP_GROUP_BYTES", group_bytes)
+    for mode in ("stochastic_rounding", "fp31_master"):
+        ref_model, _ = run_reference_adam(mode, steps=3, ga=2)
+        model, _ = run_offload_adam(mode, steps=3, ga=2)
+        assert_same_params(ref_model, model)
+
+
+def test_backward_alone_completes_the_step(fixed_seed):
+    """Hook mode: the step happens inside backward().  A loop that never calls
+    step(), zero_grad() or touches ready_for_optimizer_step again still has every
+    parameter stepped when backward() returns (the last group is closed by a
+    callback on the autograd engine, not by the next call into the optimizer)."""
+    from offload_adam_amd import Adam, OffloadAdam
+
+    data = batches(4)
+    ref = make_model(0)
+    ref_opt = Adam(ref.parameters(), mode="fp31_master", lr=1e-2, weight_decay=0.01)
+    for ids in data:
+        loss_of(ref, ids).backward()
+        ref_opt.step()
+        ref_opt.zero_grad(set_to_none=True)
+    model = make_model(0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, weight_decay=0.01,
+                          inplace_param_threshold=5000)
+    opt.ready_for_optimizer_step = True
+    for ids in data:
+        loss_of(model, ids).backward()
+        assert not opt._pending_steps and not opt._pending_inplace
+        assert all(st["step"] > 0 for st in opt.state.values())
+    torch.cuda.synchronize()
+    assert_same_params(ref, model)
+
+
+def test_hooks_called_outside_backward_step_at_once(fixed_seed):
+    """A gradient hook invoked by hand (no backward pass is running, so there is no
+    engine to call back): the parameter is stepped before the hook returns."""
+    from offload_adam_amd import OffloadAdam
+
+    model = make_model(0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode="stochastic_rounding", lr=1e-2, inplace_param_threshold=5000)
+    opt.ready_for_optimizer_step = True
+    p = opt._offload_params[0]
+    before = p.detach().clone()
+    p.grad = torch.full_like(p, 0.01)
+    opt._grad_hook(p)
+    torch.cuda.synchronize()
+    assert opt.state[p]["step"] == 1 and not opt._pending_steps
+    assert not torch.equal(before, p.detach())
+
+
 def test_transfer_streams_are_picked_by_measured_concurrency():
     """With more live streams than hardware queues, the optimizer still ends up
     with side streams whose copies run beside each other and beside kernels."""
