@@ -201,16 +201,17 @@ def link_bytes_per_step(opt, grad_accum):
     n = sum(p.numel() for p in opt._offload_params)
     state_b = sum(torch.empty(0, dtype=d).element_size()
                   for k, d in opt.offload_config.items() if k != "grad")
+    # states and gradients kept on the GPU after their write-back are not fetched again
+    states_in = state_b * sum(p.numel() for p in opt._offload_params
+                              if p not in opt._state_cached)
     if not opt.offload_grads:
-        h2d = d2h = n * state_b
-        return h2d, d2h
-    # gradients kept on the GPU after their write-back are never fetched again
+        return states_in, n * state_b
     fetched = sum(p.numel() for p in opt._offload_params if p not in opt._grad_cached)
     if opt._step_in_backward:
-        h2d = n * state_b + fetched * 2 * (grad_accum - 1)
+        h2d = states_in + fetched * 2 * (grad_accum - 1)
         d2h = n * (2 * (grad_accum - 1) + state_b)
     else:
-        h2d = n * state_b + fetched * 2 * grad_accum
+        h2d = states_in + fetched * 2 * grad_accum
         d2h = n * (2 * grad_accum + state_b)
     return h2d, d2h
 
@@ -349,13 +350,17 @@ def run(args):
                           decoupled_weight_decay=True, offload_grads=not args.grads_on_device,
                           prefetch_bytes=int(args.prefetch_gib * 2**30) if args.prefetch_gib else None,
                           grad_cache_bytes=(None if args.grad_cache_gib is None
-                                            else int(args.grad_cache_gib * 2**30)))
+                                            else int(args.grad_cache_gib * 2**30)),
+                          state_cache_bytes=(None if args.state_cache_gib is None
+                                             else int(args.state_cache_gib * 2**30)))
     torch.cuda.synchronize()
     out["optimizer_init_s"] = round(time.perf_counter() - t0, 2)
     out["offloaded_params"] = len(opt._offload_params)
     out["inplace_params"] = len(opt._inplace_params)
     out["prefetch_GiB"] = round(opt._PREFETCH_BYTES / 1024**3, 2)
     out["grad_cache_GiB"] = round(sum(p.numel() for p in opt._grad_cached) * 2 / 1024**3, 2)
+    out["state_cache_GiB"] = round(
+        sum(p.numel() for p in opt._state_cached) * (opt._bytes_per_elem_in_flight - 2) / 1024**3, 2)
     out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
 
     timeline = None
@@ -441,6 +446,10 @@ def main():
                     help="OffloadAdam(grad_cache_bytes=...): HBM for gradients kept on the GPU "
                          "after their write-back (default: the optimizer's; 0 = fetch every time "
                          "like the reference)")
+    ap.add_argument("--state-cache-gib", type=float, default=None,
+                    help="OffloadAdam(state_cache_bytes=...): HBM for optimizer states kept on the "
+                         "GPU after their write-back (default: the optimizer's; 0 = none, like "
+                         "the reference)")
     ap.add_argument("--grads-on-device", action="store_true",
                     help="OffloadAdam(offload_grads=False): the gradient sum stays in HBM")
     ap.add_argument("--copy-timeline", action="store_true",

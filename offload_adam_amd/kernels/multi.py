@@ -7,9 +7,8 @@ so the GPU does not drain between them.
 """
 
 import random
-from ctypes import c_float, c_int, c_void_p
+from ctypes import c_float, c_int, c_int64, c_uint64
 
-import numpy as np
 import torch
 
 from .. import _lib
@@ -32,7 +31,12 @@ _AUX_KEY = {
 
 
 def _ptr_table(tensors):
-    return np.fromiter((t.data_ptr() for t in tensors), dtype=np.uint64, count=len(tensors))
+    """Addresses as a C array (plain ctypes: no numpy round trip per launch)."""
+    return (c_uint64 * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def _float_table(values):
+    return (c_float * len(values))(*values)
 
 
 def adam_step_multi(
@@ -82,12 +86,15 @@ def adam_step_multi(
 
     if isinstance(steps, int):
         b1h, b2h = _common.folded_betas(beta1, beta2, steps)
-        b1 = np.full(count, b1h, dtype=np.float32)
-        b2 = np.full(count, b2h, dtype=np.float32)
+        b1 = _float_table([b1h] * count)
+        b2 = _float_table([b2h] * count)
     else:
-        pairs = [_common.folded_betas(beta1, beta2, s) for s in steps]
-        b1 = np.array([a for a, _ in pairs], dtype=np.float32)
-        b2 = np.array([b for _, b in pairs], dtype=np.float32)
+        folded = {}
+        for step in steps:
+            if step not in folded:
+                folded[step] = _common.folded_betas(beta1, beta2, step)
+        b1 = _float_table([folded[step][0] for step in steps])
+        b2 = _float_table([folded[step][1] for step in steps])
 
     seed_tab = None
     rng_code = _lib.OA_RNG_X8
@@ -99,23 +106,20 @@ def adam_step_multi(
         rng_code = _lib.OA_RNG_X8 if rng == "x8" else _lib.OA_RNG_TRITON
         if seeds is None:
             seeds = [random.getrandbits(64) for _ in range(count)]
-        seed_tab = np.array([s & 0xFFFFFFFFFFFFFFFF for s in seeds], dtype=np.uint64)
+        seed_tab = (c_uint64 * count)(*[s & 0xFFFFFFFFFFFFFFFF for s in seeds])
 
     p_tab = _ptr_table(params)
     g_tab = _ptr_table([st["grad"] for st in states])
     m_tab = _ptr_table([st["exp_avg"] for st in states])
     v_tab = _ptr_table([st["exp_avg_sq"] for st in states])
     a_tab = _ptr_table([st[aux_key] for st in states]) if aux_key is not None else None
-    n_tab = np.fromiter((p.numel() for p in params), dtype=np.int64, count=count)
-
-    def addr(a):
-        return c_void_p(a.ctypes.data) if a is not None else c_void_p(None)
+    n_tab = (c_int64 * count)(*[p.numel() for p in params])
 
     lib = _lib.load()
     with _lib.device_guard(dev):
         code = lib.oa_adam_multi(
-            c_int(MODE_CODES[mode]), c_int(count), addr(p_tab), addr(g_tab), addr(m_tab),
-            addr(v_tab), addr(a_tab), addr(n_tab), addr(b1), addr(b2), addr(seed_tab),
+            c_int(MODE_CODES[mode]), c_int(count), p_tab, g_tab, m_tab,
+            v_tab, a_tab, n_tab, b1, b2, seed_tab,
             c_float(lr), c_float(weight_decay), c_float(eps),
             c_int(1 if decoupled_weight_decay else 0), c_int(rng_code), _lib.ptr(clip_coef),
             _lib.current_stream_ptr(),

@@ -230,6 +230,15 @@ class OffloadAdam(Optimizer):
             admitted in optimizer order until the budget is used.  Default: a
             tenth of the HBM that is free when the optimizer is built; ``0``
             fetches every time, like the reference.  Results are bit-identical.
+        state_cache_bytes (int, keyword-only): the same for the optimizer states:
+            HBM that may keep the device copy of a parameter's states alive
+            after the step has written them back to the host.  The host copy
+            stays current after every step; what is saved is fetching the same
+            bytes for the next step.  Parameters are admitted from the end of the
+            optimizer's order (the ones backward reaches first, whose fetch has
+            the least time to arrive).  Default: a tenth of the HBM that is free
+            when the optimizer is built; ``0`` keeps nothing, like the reference.
+            Results are bit-identical.
     """
 
     supported_modes = {
@@ -271,6 +280,7 @@ class OffloadAdam(Optimizer):
         offload_grads=True,
         prefetch_bytes=None,
         grad_cache_bytes=None,
+        state_cache_bytes=None,
     ):
         if prefetch_policy not in ("eager", "lazy"):
             raise ValueError(f"prefetch_policy must be 'eager' or 'lazy' (got {prefetch_policy!r})")
@@ -289,6 +299,8 @@ class OffloadAdam(Optimizer):
             self._PREFETCH_BYTES = int(prefetch_bytes)
         if grad_cache_bytes is not None and grad_cache_bytes < 0:
             raise ValueError("grad_cache_bytes must be >= 0")
+        if state_cache_bytes is not None and state_cache_bytes < 0:
+            raise ValueError("state_cache_bytes must be >= 0")
         # what lives in pinned host memory between steps
         self._host_config = {
             k: d for k, d in self.offload_config.items() if k != "grad" or self.offload_grads
@@ -358,6 +370,22 @@ class OffloadAdam(Optimizer):
                     break
                 budget -= nbytes
                 self._grad_cached.add(p)
+
+        # parameters whose states stay on the GPU after their write-back
+        self._state_cached = set()
+        if self._offload_params:
+            budget = state_cache_bytes
+            if budget is None:
+                dev0 = self._offload_params[0].device
+                budget = torch.cuda.mem_get_info(dev0)[0] // 10 if dev0.type == "cuda" else 0
+            per_elem = sum(torch.empty(0, dtype=d).element_size()
+                           for k, d in self.offload_config.items() if k != "grad")
+            for p in reversed(self._offload_params):
+                nbytes = p.numel() * per_elem
+                if nbytes > budget:
+                    break
+                budget -= nbytes
+                self._state_cached.add(p)
 
         self._pending_steps = []      # offloaded parameters waiting for their group's launch
         self._pending_inplace = []    # GPU-resident ones
@@ -463,6 +491,15 @@ class OffloadAdam(Optimizer):
             )
 
     def _copy_master(self, p, tensor):
+        dev = self.device_states.get(p)
+        if dev is not None:
+            # offloaded: let a write-back still under way land first, and forget any
+            # device copy (staged or cached) of the value being replaced
+            self._flush_steps()
+            event = self.d2h_events.get(p)
+            if event is not None:
+                event.synchronize()
+            dev["master_params"] = None
         self.state[p]["master_params"].copy_(tensor)
 
     def _alloc_pinned_states(self, params, numa_node):
@@ -587,9 +624,13 @@ class OffloadAdam(Optimizer):
             else:
                 _copy_async(self._host_view(p, key), buf, _lib.OA_COPY_D2H, self.d2h_stream)
             buf.record_stream(self.d2h_stream)
-            if key != "grad" or p not in self._grad_cached:
+            if not self._stays_on_device(p, key):
                 dev[key] = None
         self.d2h_events[p] = self.d2h_stream.record_event()
+
+    def _stays_on_device(self, p, key):
+        """Write-through caches: the device copy outlives its write-back."""
+        return p in (self._grad_cached if key == "grad" else self._state_cached)
 
     def _issue_d2h_many(self, items):
         """Write-back of ``keys`` of every ``(p, keys)`` behind one fence, with one
@@ -604,7 +645,7 @@ class OffloadAdam(Optimizer):
                 buf = dev[key]
                 _copy_async(self._host_view(p, key), buf, _lib.OA_COPY_D2H, d2h)
                 buf.record_stream(d2h)
-                if key != "grad" or p not in self._grad_cached:
+                if not self._stays_on_device(p, key):
                     dev[key] = None
         event = d2h.record_event()
         for p, _ in items:
@@ -677,6 +718,9 @@ class OffloadAdam(Optimizer):
     def _step_offload(self, p, group, clip_coef=None):
         dev = self.device_states[p]
         self._ensure_on_device(p, self.offload_state_keys)
+        if p in self._state_cached and p in self.d2h_events:
+            # the kernel rewrites states whose last write-back may still be reading them
+            self._compute_stream().wait_event(self.d2h_events[p])
         self._call_step_fn(p, group, dev, clip_coef)
         self._issue_d2h(p, self._non_grad_keys)
         dev["grad"] = None
@@ -707,6 +751,7 @@ class OffloadAdam(Optimizer):
             steps,
             decoupled_weight_decay=self.decoupled_weight_decay,
             clip_coef=clip_coef,
+            validate=False,  # the optimizer's own buffers
         )
         torch._foreach_zero_([t["grad"] for t in tensors])
 
@@ -765,10 +810,14 @@ class OffloadAdam(Optimizer):
         compute = self._compute_stream()
         waited = set()
         for p in params:
-            event = self.h2d_events.get(p)
-            if event is not None and id(event) not in waited:
-                compute.wait_event(event)
-                waited.add(id(event))
+            events = [self.h2d_events.get(p)]
+            if p in self._state_cached:
+                # the kernel rewrites states whose last write-back may still be reading them
+                events.append(self.d2h_events.get(p))
+            for event in events:
+                if event is not None and id(event) not in waited:
+                    compute.wait_event(event)
+                    waited.add(id(event))
         by_group = {}
         for p in params:
             state = self.state[p]
@@ -787,7 +836,7 @@ class OffloadAdam(Optimizer):
             beta1, beta2 = group["betas"]
             adam_step_multi(self.mode, ps, tensors, group["lr"], group["weight_decay"], beta1,
                             beta2, group["eps"], steps,
-                            decoupled_weight_decay=self.decoupled_weight_decay)
+                            decoupled_weight_decay=self.decoupled_weight_decay, validate=False)
         self._issue_d2h_many([(p, self._non_grad_keys) for p in params])
         for p in params:
             self.device_states[p]["grad"] = None
@@ -829,10 +878,12 @@ class OffloadAdam(Optimizer):
         if len(self._bw_prefix) != len(order) + 1:
             # bytes of device staging of order[:j], for the bisection below
             self._bw_prefix = [0]
+            grad_b = 2 if self.offload_grads else 0
+            state_b = self._bytes_per_elem_in_flight - 2
             for q in order:
-                self._bw_prefix.append(
-                    self._bw_prefix[-1] + q.numel() * self._bytes_per_elem_in_flight
-                )
+                per_elem = ((0 if q in self._state_cached else state_b)
+                            + (0 if q in self._grad_cached else grad_b))
+                self._bw_prefix.append(self._bw_prefix[-1] + q.numel() * per_elem)
         prefix = self._bw_prefix
         first = pos + 1
         # parameters j >= first are wanted while the bytes of order[first:j] stay

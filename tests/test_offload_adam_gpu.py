@@ -628,6 +628,64 @@ def test_gradient_cache_does_not_change_results(fixed_seed, mode, cache, clip):
         assert 0 < n_cached < len(opt._offload_params)
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("cache", [0, 200_000, None])
+@pytest.mark.parametrize("clip", [None, 0.05])
+def test_state_cache_does_not_change_results(fixed_seed, mode, cache, clip):
+    """state_cache_bytes = 0 (every state is fetched for every step, as in the
+    reference), a budget that admits only some parameters, and the default: same
+    bits; the host copies are current after every step."""
+    ref_model, ref_opt = run_offload_adam(mode, steps=4, ga=2, max_grad_norm=clip,
+                                          state_cache_bytes=0, grad_cache_bytes=0)
+    model, opt = run_offload_adam(mode, steps=4, ga=2, max_grad_norm=clip,
+                                  state_cache_bytes=cache)
+    assert_same_params(ref_model, model)
+    n_cached = len(opt._state_cached)
+    if cache == 0:
+        assert n_cached == 0
+    elif cache is None:
+        assert n_cached == len(opt._offload_params)
+    else:
+        assert 0 < n_cached < len(opt._offload_params)
+    for pr, p in zip(ref_model.parameters(), model.parameters()):
+        a, b = ref_opt.state[pr], opt.state[p]
+        for k in opt._non_grad_keys:
+            assert torch.equal(a[k], b[k]), k  # pinned host copies (GPU ones for small params)
+            if p in opt._state_cached:
+                assert torch.equal(opt.device_states[p][k].cpu(), b[k].cpu()), k
+
+
+def test_loading_masters_replaces_cached_device_copies(fixed_seed):
+    """load_master_state_dict after some steps: the next step starts from the
+    loaded masters, not from a device copy kept from the previous step."""
+    from offload_adam_amd import OffloadAdam
+
+    results = []
+    for cache in (0, None):
+        model = make_model(0)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            opt = OffloadAdam(model, mode="fp32_master", lr=1e-2, inplace_param_threshold=5000,
+                              state_cache_bytes=cache)
+        data = batches(3)
+        for i in range(2):
+            opt.ready_for_optimizer_step = True
+            loss_of(model, data[i]).backward()
+            opt.step()
+        new_masters = {n: torch.full_like(p, 0.25, dtype=torch.float32)
+                       for n, p in model.named_parameters()}
+        opt.load_master_state_dict(new_masters, model)
+        opt.ready_for_optimizer_step = True
+        loss_of(model, data[2]).backward()
+        opt.step()
+        torch.cuda.synchronize()
+        results.append([p.detach().clone() for p in model.parameters()])
+        big = opt._offload_params[0]
+        assert abs(opt.state[big]["master_params"].mean().item() - 0.25) < 0.05
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+
+
 def test_cached_gradient_is_also_current_on_the_host(fixed_seed):
     """One micro-batch into a window: the pinned ``state['grad']`` holds the same
     sum whether or not the device copy was kept."""
@@ -782,7 +840,9 @@ def test_prefetch_budget_does_not_change_results(fixed_seed, prefetch_bytes):
 @pytest.mark.parametrize("kw", [dict(), dict(max_grad_norm=0.05), dict(offload_grads=False),
                                 dict(prefetch_bytes=0), dict(grad_cache_bytes=0),
                                 dict(grad_cache_bytes=0, max_grad_norm=0.05),
-                                dict(grad_cache_bytes=40_000)])
+                                dict(grad_cache_bytes=40_000), dict(state_cache_bytes=0),
+                                dict(state_cache_bytes=200_000, grad_cache_bytes=0),
+                                dict(state_cache_bytes=0, grad_cache_bytes=0, prefetch_bytes=0)])
 def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monkeypatch, kw):
     """Log every H2D / kernel / D2H the optimizer issues and check, per parameter
     and state key: a key is on the device (H2D issued, not yet written back) when
@@ -850,8 +910,8 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
             for k in keys:
                 if k == "grad" and not opt.offload_grads:
                     continue
-                # a cached gradient is written back and stays on the GPU as well
-                on_device[(p, k)] = k == "grad" and p in opt._grad_cached
+                # a cached gradient or state is written back and stays on the GPU as well
+                on_device[(p, k)] = p in (opt._grad_cached if k == "grad" else opt._state_cached)
         else:
             stepped[p] += 1
             for k in opt._non_grad_keys:
