@@ -390,6 +390,8 @@ class OffloadAdam(Optimizer):
         self._pending_steps = []      # offloaded parameters waiting for their group's launch
         self._pending_inplace = []    # GPU-resident ones
         self._pending_step_bytes = 0
+        self._pending_writebacks = []  # cached gradients whose write-back waits for its group
+        self._pending_writeback_bytes = 0
         self._flush_callback_queued = False
         self.device_states = {}
         self.h2d_events = {}
@@ -755,6 +757,19 @@ class OffloadAdam(Optimizer):
         )
         torch._foreach_zero_([t["grad"] for t in tensors])
 
+    def _flush_at_end_of_backward(self):
+        """Queue ``_flush_steps`` on the autograd engine: it runs when this backward
+        pass has executed its last node, so no group is ever left waiting for a
+        hook that does not come.  False outside a backward pass."""
+        if self._flush_callback_queued:
+            return True
+        try:
+            torch.autograd.Variable._execution_engine.queue_callback(self._flush_steps)
+        except RuntimeError:
+            return False
+        self._flush_callback_queued = True
+        return True
+
     def _queue_step(self, p, inplace=False):
         """Hook path: ``p``'s gradient is complete; step it with its group."""
         if inplace:
@@ -762,18 +777,26 @@ class OffloadAdam(Optimizer):
         else:
             self._pending_steps.append(p)
         self._pending_step_bytes += p.numel() * 2
-        if not self._flush_callback_queued:
-            # runs when this backward pass has executed its last node: no group is
-            # ever left waiting for a hook that does not come
-            try:
-                torch.autograd.Variable._execution_engine.queue_callback(self._flush_steps)
-                self._flush_callback_queued = True
-            except RuntimeError:  # called outside a backward pass: nothing to wait for
-                self._flush_steps()
-                return
-        if (len(self._pending_steps) + len(self._pending_inplace) >= self._STEP_GROUP_PARAMS
+        if not self._flush_at_end_of_backward():
+            self._flush_steps()  # called by hand: nothing to wait for
+        elif (len(self._pending_steps) + len(self._pending_inplace) >= self._STEP_GROUP_PARAMS
                 or self._pending_step_bytes >= self._STEP_GROUP_BYTES):
             self._flush_steps(final=False)
+
+    def _queue_grad_writeback(self, p):
+        """An accumulated gradient that stays on the GPU (``grad_cache_bytes``) goes
+        back to the host with its group: one fence and one event for all of them."""
+        self._pending_writebacks.append(p)
+        self._pending_writeback_bytes += p.numel() * 2
+        if (not self._flush_at_end_of_backward()
+                or len(self._pending_writebacks) >= self._STEP_GROUP_PARAMS
+                or self._pending_writeback_bytes >= self._STEP_GROUP_BYTES):
+            self._flush_writebacks()
+
+    def _flush_writebacks(self):
+        params, self._pending_writebacks, self._pending_writeback_bytes = (
+            self._pending_writebacks, [], 0)
+        self._issue_d2h_many([(p, ["grad"]) for p in params])
 
     @torch.no_grad()
     def _flush_steps(self, final=True):
@@ -781,6 +804,8 @@ class OffloadAdam(Optimizer):
         multi-tensor launch per param group, one fenced write-back."""
         if final:
             self._flush_callback_queued = False
+        if self._pending_writebacks:
+            self._flush_writebacks()
         offloaded, inplace = self._pending_steps, self._pending_inplace
         if not offloaded and not inplace:
             return
@@ -911,7 +936,8 @@ class OffloadAdam(Optimizer):
         copies, so they run under that forward pass instead of waiting for the
         first backward hook."""
         self._ready_for_optimizer_step = bool(value)
-        if getattr(self, "_pending_steps", None) or getattr(self, "_pending_inplace", None):
+        if (getattr(self, "_pending_steps", None) or getattr(self, "_pending_inplace", None)
+                or getattr(self, "_pending_writebacks", None)):
             self._flush_steps()
         if not self._ready_for_optimizer_step or not hasattr(self, "_bw_order"):
             return
@@ -1006,7 +1032,10 @@ class OffloadAdam(Optimizer):
                 # first now, up to the prefetch budget.
                 self._prefetch_ahead(-1, states_too=True)
         elif self.offload_grads:
-            self._issue_d2h(p, ["grad"])
+            if p in self._grad_cached:
+                self._queue_grad_writeback(p)
+            else:
+                self._issue_d2h(p, ["grad"])
 
     @torch.no_grad()
     def _inplace_grad_hook(self, p):
@@ -1032,8 +1061,8 @@ class OffloadAdam(Optimizer):
                 "optimizer state."
             )
         self._bw_cursor = -1  # the next backward pass starts a new prefetch window
+        self._flush_steps()  # normally empty: the end of backward has flushed
         if self._step_in_backward:
-            self._flush_steps()  # normally empty: the end of backward has flushed
             return
 
         clip_coef = None
