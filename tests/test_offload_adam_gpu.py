@@ -752,6 +752,40 @@ def test_backward_alone_completes_the_step(fixed_seed):
     assert_same_params(ref, model)
 
 
+@pytest.mark.parametrize("reentrant", [False, True])
+def test_activation_checkpointing_of_either_kind(fixed_seed, reentrant):
+    """Re-entrant checkpointing runs nested backward passes (each with its own
+    end-of-pass callbacks); the result is the same as without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+
+    from offload_adam_amd import OffloadAdam
+
+    class Checkpointed(TinyNet):
+        def forward(self, ids):
+            x = self.emb(ids)
+            for b in self.blocks:
+                x = x + checkpoint(lambda y, b=b: b["down"](F.gelu(b["up"](b["norm"](y)))), x,
+                                   use_reentrant=reentrant)
+            return self.head(x)
+
+    ref_model, _ = run_offload_adam("fp31_master", steps=3, ga=2)
+    torch.manual_seed(0)
+    model = Checkpointed().to(device="cuda", dtype=BF16)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, weight_decay=0.01,
+                          inplace_param_threshold=5000)
+    data = batches(6)
+    for s_ in range(3):
+        for mb in range(2):
+            opt.ready_for_optimizer_step = mb == 1
+            loss_of(model, data[s_ * 2 + mb]).backward()
+        opt.step()
+        opt.zero_grad()
+    torch.cuda.synchronize()
+    assert_same_params(ref_model, model)
+
+
 def test_hooks_called_outside_backward_step_at_once(fixed_seed):
     """A gradient hook invoked by hand (no backward pass is running, so there is no
     engine to call back): the parameter is stepped before the hook returns."""
