@@ -387,6 +387,16 @@ class OffloadAdam(Optimizer):
                 budget -= nbytes
                 self._state_cached.add(p)
 
+        if self.verbose > 0 and self._offload_params:
+            cached_g = sum(p.numel() for p in self._grad_cached) * 2
+            cached_s = sum(p.numel() for p in self._state_cached) * (
+                sum(torch.empty(0, dtype=d).element_size()
+                    for k, d in self.offload_config.items() if k != "grad"))
+            print(f"HBM the optimizer may hold: gradient cache {cached_g / _GIB:.2f} GB "
+                  f"({len(self._grad_cached)} params), state cache {cached_s / _GIB:.2f} GB "
+                  f"({len(self._state_cached)} params), prefetch staging "
+                  f"{self._PREFETCH_BYTES / _GIB:.2f} GB")
+
         self._pending_steps = []      # offloaded parameters waiting for their group's launch
         self._pending_inplace = []    # GPU-resident ones
         self._pending_step_bytes = 0
