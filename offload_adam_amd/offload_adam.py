@@ -552,7 +552,9 @@ class OffloadAdam(Optimizer):
     #   compute stream's allocator pool);
     #   the compute stream waits for H2D(p) before touching p's device states;
     #   D2H(p) starts after everything the compute stream has enqueued so far;
-    #   a device buffer is not recycled before the D2H that reads it is done.
+    #   a device buffer is not recycled before the D2H that reads it is done;
+    #   a device buffer that outlives its D2H (gradient / state cache) is not
+    #   written again by the compute stream before that D2H is done.
 
     def _check_copy_engines(self):
         """Warn once when the fixed-engine tools library is not in effect: the HIP
