@@ -786,6 +786,20 @@ def test_activation_checkpointing_of_either_kind(fixed_seed, reentrant):
     assert_same_params(ref_model, model)
 
 
+def test_verbose_reports_pinned_memory_and_budgets(capsys):
+    from offload_adam_amd import OffloadAdam
+
+    model = make_model(0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        OffloadAdam(model, mode="fp32_master", inplace_param_threshold=5000, verbose=1,
+                    grad_cache_bytes=40_000)
+    out = capsys.readouterr().out
+    assert "Pinned host memory allocated" in out
+    assert "In-place GPU states" in out
+    assert "gradient cache" in out and "(1 params)" in out and "state cache" in out
+
+
 def test_hooks_called_outside_backward_step_at_once(fixed_seed):
     """A gradient hook invoked by hand (no backward pass is running, so there is no
     engine to call back): the parameter is stepped before the hook returns."""
