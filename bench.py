@@ -157,6 +157,47 @@ def cpu_baseline(mode, target_elems=256 * 1024 * 1024, iters=5):
     }
 
 
+def cpu_baselines_of_the_other_kernels(rows=512, cols=14336):
+    """The C restatement (one thread) of every kernel besides the AdamW update,
+    on a bounded sample: ``rows`` x ``cols`` of the codec workload's weight and as
+    many elements of gradient.  GB/s of the same algorithmic bytes the GPU figures
+    of bench_kernels.py use (bf16 source and output)."""
+    import numpy as np
+
+    import oracle
+
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)
+    x[rng.random((rows, cols)) < 0.01] *= 10
+    # the values a bf16 weight holds
+    x = (oracle.narrow_array(x, "bfloat16").astype(np.uint32) << 16).view(np.float32)
+    x = np.ascontiguousarray(x.reshape(rows, cols))
+    n = rows * cols
+    g_bits = oracle.narrow_array((rng.standard_normal(n) * 5e-3).astype(np.float32), "bfloat16")
+    out = {}
+
+    def timed(name, alg_bytes, fn):
+        fn()
+        t0 = time.perf_counter()
+        res = fn()
+        dt = time.perf_counter() - t0
+        out[name] = round(alg_bytes / dt / 1e9, 3)
+        return res
+
+    timed("grad_norm", 2 * n, lambda: oracle.grad_norm_bf16(g_bits))
+    q8 = timed("quant_int8", 3 * n, lambda: oracle.quant_int8(x))
+    timed("dequant_int8", 3 * n, lambda: oracle.dequant_int8(*q8))
+    q4 = timed("quant_int4", n * (2 + 0.5 + 2 / 128), lambda: oracle.quant_int4(x, 128))
+    timed("dequant_int4", n * (2 + 0.5 + 2 / 128), lambda: oracle.dequant_int4(*q4, 128))
+    qn = timed("quant_nf4", n * (2 + 0.5 + 4 / 64), lambda: oracle.quant_nf4(x, 64))
+    timed("dequant_nf4", n * (2 + 0.5 + 4 / 64), lambda: oracle.dequant_nf4(*qn, 64))
+    qf = timed("quant_nvfp4", n * (4 + 0.5 + 1 / 16), lambda: oracle.quant_nvfp4(x))
+    timed("dequant_nvfp4", n * (2 + 0.5 + 1 / 16), lambda: oracle.dequant_nvfp4(*qf))
+    return {"unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{rows} x {cols} elements per kernel, C restatement, one pass timed",
+            "value": out}
+
+
 def offloaded_step_8b(timeout_s=420):
     """The second half of the metric: step time of a synthetic Llama-3-8B-shaped
     training step through OffloadAdam (benchmark config 4), measured by
@@ -196,6 +237,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run three 1 GiB device copies first (reference for counter runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-baseline-other-kernels", action="store_true",
+                    help="also time the CPU restatement of the norm and codec kernels "
+                         "(bounded sample, a few seconds) and add it to the line")
     ap.add_argument("--no-e2e", action="store_true",
                     help="skip the 8B offloaded training step (bench_e2e.py, run as a child "
                          "process after the timed region; about a minute)")
@@ -342,6 +386,8 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(mode)
+    if args.cpu_baseline_other_kernels:
+        out["cpu_baseline_other_kernels"] = cpu_baselines_of_the_other_kernels()
     if not args.no_e2e and args.workload == "c1_sr_llama1b":
         del tensors, p_list, st_list
         torch.cuda.empty_cache()
