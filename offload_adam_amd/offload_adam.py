@@ -777,7 +777,7 @@ class OffloadAdam(Optimizer):
             return True
         try:
             torch.autograd.Variable._execution_engine.queue_callback(self._flush_steps)
-        except RuntimeError:
+        except (RuntimeError, AttributeError):  # no pass running / no such engine hook
             return False
         self._flush_callback_queued = True
         return True
