@@ -434,13 +434,16 @@ inline dim3 i4_grid(unsigned row_tiles, unsigned groups) {
 // along the row index, which is the contiguous direction of the transposed
 // (cols/8, rows) storage.  (Issuing the encoder's four row passes together, or a
 // 128-row encoder tile, measured 10-15 % slower than this plain loop.)
-template <int SRC>
+// WPR = words per (row, group) when it is known at compile time (the usual
+// group sizes 128, 64 and 32): every index division below folds into shifts and
+// the row passes unroll; 0 = take it from `group` at run time.
+template <int SRC, int WPR>
 __global__ void __launch_bounds__(kT)
 quant_int4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int group,
                   int32_t* __restrict__ qweight, void* __restrict__ scales, int sdt,
                   const AdamSrc ad) {
   extern __shared__ uint32_t i4_lds[];
-  const int wpr = group >> 3;
+  const int wpr = WPR ? WPR : (group >> 3);
   uint32_t* words = i4_lds;                                  // [wpr][kI4RowsQ + 1]
   float* scale_s = reinterpret_cast<float*>(words + wpr * (kI4RowsQ + 1));
 #if OA_I4_GROUP_FASTEST
@@ -477,13 +480,13 @@ quant_int4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, in
     store_scale(scales, sdt, gi * rows + r0 + threadIdx.x, scale_s[threadIdx.x]);
 }
 
-template <int OUT>
+template <int OUT, int WPR>
 __global__ void __launch_bounds__(kT)
 dequant_int4_kernel(const int32_t* __restrict__ qweight, const void* __restrict__ scales,
                     int sdt, int64_t rows, int group, void* __restrict__ out,
                     int64_t ostride) {
   extern __shared__ uint32_t i4_lds[];
-  const int wpr = group >> 3;
+  const int wpr = WPR ? WPR : (group >> 3);
   uint32_t* words = i4_lds;
   float* scale_s = reinterpret_cast<float*>(words + wpr * (kI4RowsD + 1));
 #if OA_I4_GROUP_FASTEST
@@ -677,11 +680,15 @@ __device__ __forceinline__ uint32_t nf4_pack8(const float (&x)[8], float inv16, 
 }
 
 // Flat over octets; lpg = block/8 lanes share a block (power of two <= 64).
-template <int SRC>
+// LPG != 0: that many lanes per block, known at compile time (8 = the usual
+// 64-element block): the shuffle ladder of the block maximum unrolls.
+template <int SRC, int LPG>
 __global__ void __launch_bounds__(kT)
 quant_nf4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int64_t cols,
-                 int lpg, int lpg_shift, uint32_t* __restrict__ packed,
+                 int lpg_arg, int lpg_shift_arg, uint32_t* __restrict__ packed,
                  float* __restrict__ absmax_out, int mode, const AdamSrc ad) {
+  const int lpg = LPG ? LPG : lpg_arg;
+  const int lpg_shift = LPG ? __builtin_ctz((unsigned)(LPG ? LPG : 1)) : lpg_shift_arg;
   // The fused AdamW source moves 18 bytes per element: one octet per lane and the
   // XCD-aware tile order of the step kernels suit it better than four in flight.
   constexpr int kOct = SRC == kSrcAdam ? 1 : oa::kOct;
@@ -1072,6 +1079,14 @@ inline bool rows_vec(const void* p, int dt, int64_t stride, int64_t cols) {
   return cols % 8 == 0 && aligned_to(p, 16) && (stride * esize(dt)) % 16 == 0;
 }
 
+#define OA_DISPATCH_WPR(wpr, CALL)                    \
+  switch (wpr) {                                      \
+    case 16: { constexpr int W = 16; CALL; break; }   \
+    case 8: { constexpr int W = 8; CALL; break; }     \
+    case 4: { constexpr int W = 4; CALL; break; }     \
+    default: { constexpr int W = 0; CALL; break; }    \
+  }
+
 #define OA_DISPATCH_DT(dt, CALL)                      \
   switch (dt) {                                       \
     case OA_F32: { constexpr int DT = OA_F32; CALL; break; }   \
@@ -1149,11 +1164,11 @@ extern "C" int oa_quant_int4(const void* src, int src_dtype, int64_t src_row_str
     const int wpr = (int)(group / 8);
     const size_t lds = (size_t)wpr * (kI4RowsQ + 1) * 4 + kI4RowsQ * 4;
     const dim3 grid = i4_grid((unsigned)((rows + kI4RowsQ - 1) / kI4RowsQ), (unsigned)ng);
-    OA_DISPATCH_DT(src_dtype,
-                   hipLaunchKernelGGL(quant_int4_kernel<DT>, grid, dim3(kT), lds, s, src,
-                                      src_row_stride, rows, (int)group,
-                                      static_cast<int32_t*>(qweight), scales, scale_dtype,
-                                      AdamSrc{}));
+    OA_DISPATCH_DT(src_dtype, OA_DISPATCH_WPR(
+        wpr, hipLaunchKernelGGL((quant_int4_kernel<DT, W>), grid, dim3(kT), lds, s, src,
+                                src_row_stride, rows, (int)group,
+                                static_cast<int32_t*>(qweight), scales, scale_dtype,
+                                AdamSrc{})));
   } else {
     OA_DISPATCH_DT(src_dtype,
                    hipLaunchKernelGGL(quant_int4_generic<DT>, dim3(blocks_for(rows * ng)),
@@ -1182,10 +1197,10 @@ extern "C" int oa_dequant_int4(const void* qweight, const void* scales, int scal
     const int wpr = (int)(group / 8);
     const size_t lds = (size_t)wpr * (kI4RowsD + 1) * 4 + kI4RowsD * 4;
     const dim3 grid = i4_grid((unsigned)((rows + kI4RowsD - 1) / kI4RowsD), (unsigned)ng);
-    OA_DISPATCH_DT(out_dtype,
-                   hipLaunchKernelGGL(dequant_int4_kernel<DT>, grid, dim3(kT), lds, s,
-                                      static_cast<const int32_t*>(qweight), scales, scale_dtype,
-                                      rows, (int)group, out, out_row_stride));
+    OA_DISPATCH_DT(out_dtype, OA_DISPATCH_WPR(
+        wpr, hipLaunchKernelGGL((dequant_int4_kernel<DT, W>), grid, dim3(kT), lds, s,
+                                static_cast<const int32_t*>(qweight), scales, scale_dtype,
+                                rows, (int)group, out, out_row_stride)));
   } else {
     OA_DISPATCH_DT(out_dtype,
                    hipLaunchKernelGGL(dequant_int4_generic<DT>,
@@ -1210,7 +1225,7 @@ extern "C" int oa_quant_nf4(const void* src, int src_dtype, int64_t src_row_stri
                     pow2(block / 8) && block <= 512 && aligned_to(packed, 4);
   if (fast) {
     OA_DISPATCH_DT(src_dtype,
-                   hipLaunchKernelGGL(quant_nf4_kernel<DT>, dim3(blocks_oct(rows * (cols / 8))),
+                   hipLaunchKernelGGL((block == 64 ? quant_nf4_kernel<DT, 8> : quant_nf4_kernel<DT, 0>), dim3(blocks_oct(rows * (cols / 8))),
                                       dim3(kT), 0, s, src, src_row_stride, rows, cols,
                                       (int)(block / 8), log2i(block / 8),
                                       static_cast<uint32_t*>(packed), static_cast<float*>(absmax),
@@ -1415,9 +1430,10 @@ extern "C" int oa_adam_requant_int4(const void* grad, void* exp_avg, void* exp_a
   const int wpr = (int)(group / 8);
   const size_t lds = (size_t)wpr * (kI4RowsQ + 1) * 4 + kI4RowsQ * 4;
   const dim3 grid = i4_grid((unsigned)((rows + kI4RowsQ - 1) / kI4RowsQ), (unsigned)(cols / group));
-  hipLaunchKernelGGL(quant_int4_kernel<kSrcAdam>, grid, dim3(kT), lds,
-                     static_cast<hipStream_t>(stream), nullptr, cols, rows, (int)group,
-                     static_cast<int32_t*>(qweight), scales, scale_dtype, ad);
+  OA_DISPATCH_WPR(wpr, hipLaunchKernelGGL((quant_int4_kernel<kSrcAdam, W>), grid, dim3(kT), lds,
+                                          static_cast<hipStream_t>(stream), nullptr, cols, rows,
+                                          (int)group, static_cast<int32_t*>(qweight), scales,
+                                          scale_dtype, ad));
   return launch_status();
 }
 
@@ -1435,7 +1451,8 @@ extern "C" int oa_adam_requant_nf4(const void* grad, void* exp_avg, void* exp_av
   if (!pow2(block / 8) || block > 512) return OA_EINVAL;
   if (!packed || !absmax) return OA_EINVAL;
   if (!aligned_to(packed, 4) || !aligned_to(absmax, 4)) return OA_EALIGN;
-  hipLaunchKernelGGL(quant_nf4_kernel<kSrcAdam>, dim3(xcd_grid(blocks_for(rows * (cols / 8)))),
+  hipLaunchKernelGGL((block == 64 ? quant_nf4_kernel<kSrcAdam, 8> : quant_nf4_kernel<kSrcAdam, 0>),
+                     dim3(xcd_grid(blocks_for(rows * (cols / 8)))),
                      dim3(kT), 0, static_cast<hipStream_t>(stream), nullptr, cols, rows, cols,
                      (int)(block / 8), log2i(block / 8), static_cast<uint32_t*>(packed),
                      static_cast<float*>(absmax), kFlat, ad);
