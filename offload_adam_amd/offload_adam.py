@@ -765,7 +765,6 @@ class OffloadAdam(Optimizer):
             steps,
             decoupled_weight_decay=self.decoupled_weight_decay,
             clip_coef=clip_coef,
-            validate=False,  # the optimizer's own buffers
         )
         torch._foreach_zero_([t["grad"] for t in tensors])
 
@@ -861,8 +860,11 @@ class OffloadAdam(Optimizer):
             state["step"] += 1
             group = self._param2group[p]
             dev = self.device_states[p]
-            if p in self._quant_params or not (p.data.is_contiguous() and p.dtype == _BF16):
-                self._call_step_fn(p, group, dev)  # its own launch (re-encodes the payload)
+            if (p in self._quant_params or p.dtype != _BF16 or not p.data.is_contiguous()
+                    or not dev["grad"].is_contiguous() or dev["grad"].dtype != _BF16):
+                # its own launch: a quantised weight is re-encoded there, and anything
+                # the kernels cannot take is reported by the step function's checks
+                self._call_step_fn(p, group, dev)
             else:
                 by_group.setdefault(id(group), (group, [], [], []))
                 _, ps, tensors, steps = by_group[id(group)]

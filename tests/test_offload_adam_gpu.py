@@ -973,3 +973,23 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
     written_back = {(p, k) for op, p, keys in log[last_step_index:] if op == "d2h" for k in keys}
     p_last = log[last_step_index][1]
     assert {(p_last, k) for k in opt._non_grad_keys} <= written_back
+
+
+def test_parameters_the_kernels_cannot_take_are_reported():
+    """fp32 parameters: the step function's checks raise instead of the grouped
+    launch reading them as bf16."""
+    from offload_adam_amd import OffloadAdam
+
+    for threshold in (0, 10**9):  # everything offloaded / everything GPU-resident
+        torch.manual_seed(0)
+        model = TinyNet().to(device="cuda", dtype=torch.float32)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            opt = OffloadAdam(model, mode="stochastic_rounding", inplace_param_threshold=threshold)
+        opt.ready_for_optimizer_step = True
+        ids = batches(1)[0]
+        with pytest.raises((TypeError, RuntimeError)):
+            F.cross_entropy(model(ids).reshape(-1, 50), ids.reshape(-1)).backward()
+            opt.step()
+        opt._pending_steps.clear()
+        opt._pending_inplace.clear()
