@@ -402,7 +402,6 @@ class OffloadAdam(Optimizer):
         self._pending_step_bytes = 0
         self._pending_writebacks = []  # cached gradients whose write-back waits for its group
         self._pending_writeback_bytes = 0
-        self._flush_callback_queued = False
         self.device_states = {}
         self.h2d_events = {}
         self.d2h_events = {}
@@ -771,14 +770,16 @@ class OffloadAdam(Optimizer):
     def _flush_at_end_of_backward(self):
         """Queue ``_flush_steps`` on the autograd engine: it runs when this backward
         pass has executed its last node, so no group is ever left waiting for a
-        hook that does not come.  False outside a backward pass."""
-        if self._flush_callback_queued:
-            return True
+        hook that does not come.  False outside a backward pass.
+
+        Queued once per parameter (half a microsecond; a call that finds nothing
+        pending returns at once) rather than once per pass behind a flag: a pass
+        that raises never runs its callbacks, and a flag it left set would keep
+        the next pass from queueing its own."""
         try:
             torch.autograd.Variable._execution_engine.queue_callback(self._flush_steps)
         except (RuntimeError, AttributeError):  # no pass running / no such engine hook
             return False
-        self._flush_callback_queued = True
         return True
 
     def _queue_step(self, p, inplace=False):
@@ -792,7 +793,7 @@ class OffloadAdam(Optimizer):
             self._flush_steps()  # called by hand: nothing to wait for
         elif (len(self._pending_steps) + len(self._pending_inplace) >= self._STEP_GROUP_PARAMS
                 or self._pending_step_bytes >= self._STEP_GROUP_BYTES):
-            self._flush_steps(final=False)
+            self._flush_steps()
 
     def _queue_grad_writeback(self, p):
         """An accumulated gradient that stays on the GPU (``grad_cache_bytes``) goes
@@ -810,11 +811,9 @@ class OffloadAdam(Optimizer):
         self._issue_d2h_many([(p, ["grad"]) for p in params])
 
     @torch.no_grad()
-    def _flush_steps(self, final=True):
+    def _flush_steps(self):
         """Step every queued parameter: fetch what is missing (one fence), one
         multi-tensor launch per param group, one fenced write-back."""
-        if final:
-            self._flush_callback_queued = False
         if self._pending_writebacks:
             self._flush_writebacks()
         offloaded, inplace = self._pending_steps, self._pending_inplace
@@ -1039,7 +1038,7 @@ class OffloadAdam(Optimizer):
         if self._step_in_backward and last:
             self._queue_step(p)
             if self._bw_order_known and pos == len(self._bw_order) - 1:
-                self._flush_steps(final=False)
+                self._flush_steps()
                 # The step is complete.  The host->device direction is idle until
                 # the next accumulation pass needs gradients back (never, with
                 # offload_grads=False): stage the states the next step touches

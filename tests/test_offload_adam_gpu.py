@@ -993,3 +993,39 @@ def test_parameters_the_kernels_cannot_take_are_reported():
             opt.step()
         opt._pending_steps.clear()
         opt._pending_inplace.clear()
+
+
+def test_a_backward_pass_that_raises_does_not_stall_later_ones(fixed_seed):
+    """A pass that raises midway never reaches its end-of-pass callbacks.  The passes
+    after it still close their last group by themselves (no step(), no flag
+    toggling in between)."""
+    from offload_adam_amd import OffloadAdam
+
+    class Boom(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            return x.clone()
+
+        @staticmethod
+        def backward(ctx, g):
+            raise RuntimeError("boom")
+
+    model = make_model(0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, inplace_param_threshold=5000)
+    opt.ready_for_optimizer_step = True
+    ids = batches(1)[0]
+    x = model.emb(ids)
+    for i, b in enumerate(model.blocks):
+        if i == 1:
+            x = Boom.apply(x)  # head and the last block get their gradients, then it raises
+        x = x + b["down"](F.gelu(b["up"](b["norm"](x))))
+    with pytest.raises(RuntimeError, match="boom"):
+        F.cross_entropy(model.head(x).float().reshape(-1, 50), ids.reshape(-1)).backward()
+    for ids in batches(3, seed=2):
+        loss_of(model, ids).backward()
+        assert not opt._pending_steps and not opt._pending_inplace
+    torch.cuda.synchronize()
+    steps = {st["step"] for st in opt.state.values()}
+    assert min(steps) >= 3
