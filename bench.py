@@ -218,7 +218,7 @@ def offloaded_step_8b(timeout_s=420):
     keep = ("model", "mode", "steps", "warmup", "seq", "grad_accum", "offload_grads", "params", "step_s",
             "tokens_per_s", "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step",
             "d2h_GB_per_step", "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak",
-            "link_floor_s", "pinned_GiB", "prefetch_GiB", "grad_cache_GiB", "state_cache_GiB", "peak_gpu_GiB", "optimizer_init_s", "copy_engines",
+            "link_floor_s", "pinned_GiB", "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB", "peak_gpu_GiB", "optimizer_init_s", "copy_engines",
             "transfer_streams")
     return {k: full[k] for k in keep if k in full}
 

@@ -207,12 +207,12 @@ def link_bytes_per_step(opt, grad_accum):
     if not opt.offload_grads:
         return states_in, n * state_b
     fetched = sum(p.numel() for p in opt._offload_params if p not in opt._grad_cached)
-    if opt._step_in_backward:
-        h2d = states_in + fetched * 2 * (grad_accum - 1)
-        d2h = n * (2 * (grad_accum - 1) + state_b)
-    else:
-        h2d = states_in + fetched * 2 * grad_accum
-        d2h = n * (2 * grad_accum + state_b)
+    # partial sums written to the host: all of them, or (write-back gradient cache)
+    # only those that do not stay on the GPU
+    written = fetched if opt._grad_cache_write_back else n
+    passes = grad_accum - 1 if opt._step_in_backward else grad_accum
+    h2d = states_in + fetched * 2 * passes
+    d2h = n * state_b + written * 2 * passes
     return h2d, d2h
 
 
@@ -352,13 +352,15 @@ def run(args):
                           grad_cache_bytes=(None if args.grad_cache_gib is None
                                             else int(args.grad_cache_gib * 2**30)),
                           state_cache_bytes=(None if args.state_cache_gib is None
-                                             else int(args.state_cache_gib * 2**30)))
+                                             else int(args.state_cache_gib * 2**30)),
+                          grad_cache_policy=args.grad_cache_policy)
     torch.cuda.synchronize()
     out["optimizer_init_s"] = round(time.perf_counter() - t0, 2)
     out["offloaded_params"] = len(opt._offload_params)
     out["inplace_params"] = len(opt._inplace_params)
     out["prefetch_GiB"] = round(opt._PREFETCH_BYTES / 1024**3, 2)
     out["grad_cache_GiB"] = round(sum(p.numel() for p in opt._grad_cached) * 2 / 1024**3, 2)
+    out["grad_cache_policy"] = args.grad_cache_policy
     out["state_cache_GiB"] = round(
         sum(p.numel() for p in opt._state_cached) * (opt._bytes_per_elem_in_flight - 2) / 1024**3, 2)
     out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
@@ -450,6 +452,10 @@ def main():
                     help="OffloadAdam(state_cache_bytes=...): HBM for optimizer states kept on the "
                          "GPU after their write-back (default: the optimizer's; 0 = none, like "
                          "the reference)")
+    ap.add_argument("--grad-cache-policy", default="write_back",
+                    choices=["write_back", "write_through"],
+                    help="OffloadAdam(grad_cache_policy=...): 'write_through' sends every partial "
+                         "gradient sum to the host after its micro-batch, like the reference")
     ap.add_argument("--grads-on-device", action="store_true",
                     help="OffloadAdam(offload_grads=False): the gradient sum stays in HBM")
     ap.add_argument("--copy-timeline", action="store_true",

@@ -230,6 +230,14 @@ class OffloadAdam(Optimizer):
             admitted in optimizer order until the budget is used.  Default: a
             tenth of the HBM that is free when the optimizer is built; ``0``
             fetches every time, like the reference.  Results are bit-identical.
+        grad_cache_policy (str, keyword-only): when a gradient kept by
+            ``grad_cache_bytes`` reaches the host.  ``'write_back'`` (default):
+            when somebody asks for it - ``state_dict()`` brings every host
+            gradient up to date before it returns - so partial sums that the next
+            micro-batch replaces anyway do not cross the link at all.
+            ``'write_through'``: after every micro-batch, as the reference does,
+            for code that reads ``optimizer.state[p]['grad']`` directly between
+            micro-batches.
         state_cache_bytes (int, keyword-only): the same for the optimizer states:
             HBM that may keep the device copy of a parameter's states alive
             after the step has written them back to the host.  The host copy
@@ -281,6 +289,7 @@ class OffloadAdam(Optimizer):
         prefetch_bytes=None,
         grad_cache_bytes=None,
         state_cache_bytes=None,
+        grad_cache_policy="write_back",
     ):
         if prefetch_policy not in ("eager", "lazy"):
             raise ValueError(f"prefetch_policy must be 'eager' or 'lazy' (got {prefetch_policy!r})")
@@ -301,6 +310,10 @@ class OffloadAdam(Optimizer):
             raise ValueError("grad_cache_bytes must be >= 0")
         if state_cache_bytes is not None and state_cache_bytes < 0:
             raise ValueError("state_cache_bytes must be >= 0")
+        if grad_cache_policy not in ("write_back", "write_through"):
+            raise ValueError("grad_cache_policy must be 'write_back' or 'write_through' "
+                             f"(got {grad_cache_policy!r})")
+        self._grad_cache_write_back = grad_cache_policy == "write_back"
         # what lives in pinned host memory between steps
         self._host_config = {
             k: d for k, d in self.offload_config.items() if k != "grad" or self.offload_grads
@@ -357,8 +370,9 @@ class OffloadAdam(Optimizer):
                 free, _ = torch.cuda.mem_get_info(dev0)
                 self._PREFETCH_BYTES = max(2 << 30, free // 10)
 
-        # parameters whose accumulated gradient stays on the GPU after its write-back
+        # parameters whose accumulated gradient stays on the GPU between micro-batches
         self._grad_cached = set()
+        self._stale_host_grads = set()  # write_back policy: host copy older than the device's
         if self.offload_grads and self._offload_params:
             budget = grad_cache_bytes
             if budget is None:
@@ -685,12 +699,21 @@ class OffloadAdam(Optimizer):
             else:
                 dev["grad"].add_(p.grad)
         elif state["host_grad_valid"]:
-            if dev.get("grad") is not None and p in self.d2h_events:
-                # the device copy was kept (grad_cache_bytes): its write-back to the
-                # host must have read it before the sum below overwrites it
-                self._compute_stream().wait_event(self.d2h_events[p])
-            self._ensure_on_device(p, ["grad"])
-            dev["grad"].add_(p.grad)
+            kept = dev.get("grad")
+            if kept is not None and kept.dtype == p.grad.dtype and p.grad.is_contiguous():
+                # The device copy was kept (grad_cache_bytes) and its write-back may
+                # still be reading it.  The sum goes into this micro-batch's buffer
+                # instead (a + b == b + a bit for bit), so the compute stream never
+                # waits for the host link; the kept buffer is released when the
+                # write-back that holds it (record_stream) is done.
+                p.grad.add_(kept)
+                dev["grad"] = p.grad
+            else:
+                if kept is not None and p in self.d2h_events:
+                    # in-place sum: the write-back must have read the kept copy first
+                    self._compute_stream().wait_event(self.d2h_events[p])
+                self._ensure_on_device(p, ["grad"])
+                dev["grad"].add_(p.grad)
         else:
             dev["grad"] = p.grad
             state["host_grad_valid"] = True
@@ -737,6 +760,7 @@ class OffloadAdam(Optimizer):
         self._call_step_fn(p, group, dev, clip_coef)
         self._issue_d2h(p, self._non_grad_keys)
         dev["grad"] = None
+        self._stale_host_grads.discard(p)
 
     def _step_inplace(self, p, group, clip_coef=None):
         state = self.state[p]
@@ -879,6 +903,7 @@ class OffloadAdam(Optimizer):
         for p in params:
             self.device_states[p]["grad"] = None
             self.state[p]["host_grad_valid"] = False
+        self._stale_host_grads.difference_update(params)
 
     def _record_grad_norm(self, p, grad):
         grad_clip.grad_norm_(grad.reshape(-1), self.state[p]["grad_norm"])
@@ -1045,10 +1070,12 @@ class OffloadAdam(Optimizer):
                 # first now, up to the prefetch budget.
                 self._prefetch_ahead(-1, states_too=True)
         elif self.offload_grads:
-            if p in self._grad_cached:
-                self._queue_grad_writeback(p)
-            else:
+            if p not in self._grad_cached:
                 self._issue_d2h(p, ["grad"])
+            elif self._grad_cache_write_back:
+                self._stale_host_grads.add(p)
+            else:
+                self._queue_grad_writeback(p)
 
     @torch.no_grad()
     def _inplace_grad_hook(self, p):
@@ -1117,9 +1144,19 @@ class OffloadAdam(Optimizer):
 
     def state_dict(self):
         """``Optimizer.state_dict()``; parameters still waiting for their group's
-        launch are stepped first."""
+        launch are stepped first, and host gradients that the ``'write_back'``
+        gradient cache has let fall behind are brought up to date."""
         self._flush_steps()
+        self._refresh_host_grads()
         return super().state_dict()
+
+    def _refresh_host_grads(self):
+        stale = [p for p in self._stale_host_grads
+                 if self.device_states[p].get("grad") is not None]
+        self._stale_host_grads.clear()
+        if stale:
+            self._issue_d2h_many([(p, ["grad"]) for p in stale])
+            self.d2h_events[stale[0]].synchronize()
 
     @torch.no_grad()
     def load_master_state_dict(self, state_dict, model, strict=False):
@@ -1224,6 +1261,7 @@ class OffloadAdam(Optimizer):
                 dev[name] = None
         self.h2d_events.clear()
         self.d2h_events.clear()
+        self._stale_host_grads.clear()
         self._bw_cursor = -1
         self._bw_issued_upto = 0
         for key, p in pairs:

@@ -520,6 +520,8 @@ def test_resume_continues_bit_identically(fixed_seed, mode, ga, save_after_micro
         a, b = ref_opt.state[pr], opt2.state[p2]
         assert set(a) == set(b)
         for k in a:
+            if k == "grad" and a.get("host_grad_valid") is False:
+                continue  # no window is open: the host gradient holds no information
             if isinstance(a[k], torch.Tensor):
                 assert torch.equal(a[k].cpu(), b[k].cpu()), k
             else:
@@ -607,17 +609,21 @@ def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("cache", [0, 40_000, None])
 @pytest.mark.parametrize("clip", [None, 0.05])
-def test_gradient_cache_does_not_change_results(fixed_seed, mode, cache, clip):
+@pytest.mark.parametrize("policy", ["write_back", "write_through"])
+def test_gradient_cache_does_not_change_results(fixed_seed, mode, cache, clip, policy):
     """grad_cache_bytes = 0 (every accumulated gradient is fetched back, as in the
-    reference), a budget that admits only some parameters, and the default: same
-    bits as the optimizer without offloading, on the hook path and the clip path;
-    the host copy of the gradient sum is current in every case."""
+    reference), a budget that admits only some parameters, and the default, under
+    either write policy: same bits as the optimizer without offloading, on the
+    hook path and the clip path."""
+    if cache == 0 and policy == "write_through":
+        pytest.skip("nothing is cached: the policy has nothing to decide")
     if clip is None:
         ref_model, _ = run_reference_adam(mode, steps=3, ga=3)
     else:
         ref_model, _ = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip,
                                         grad_cache_bytes=0)
-    model, opt = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip, grad_cache_bytes=cache)
+    model, opt = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip, grad_cache_bytes=cache,
+                                  grad_cache_policy=policy)
     assert_same_params(ref_model, model)
     n_cached = len(opt._grad_cached)
     if cache == 0:
@@ -686,28 +692,46 @@ def test_loading_masters_replaces_cached_device_copies(fixed_seed):
         assert torch.equal(a, b)
 
 
-def test_cached_gradient_is_also_current_on_the_host(fixed_seed):
-    """One micro-batch into a window: the pinned ``state['grad']`` holds the same
-    sum whether or not the device copy was kept."""
+def test_cached_gradient_reaches_the_host(fixed_seed):
+    """Two micro-batches into a window, the pinned ``state['grad']`` holds the same
+    sum whether or not the device copy was kept: at once under 'write_through',
+    and in what ``state_dict()`` returns under 'write_back' (where nothing crossed
+    the link before that call)."""
     from offload_adam_amd import OffloadAdam
 
     sums = []
-    for cache in (0, None):
+    for cache, policy in ((0, "write_back"), (None, "write_through"), (None, "write_back")):
         model = make_model(0)
         with warnings.catch_warnings():
             warnings.simplefilter("ignore")
             opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, inplace_param_threshold=5000,
-                              grad_cache_bytes=cache)
+                              grad_cache_bytes=cache, grad_cache_policy=policy)
         data = batches(2)
         for mb in range(2):
             opt.ready_for_optimizer_step = False
             loss_of(model, data[mb]).backward()
         torch.cuda.synchronize()
-        sums.append([opt.state[p]["grad"].clone() for p in opt._offload_params])
+        lazy = cache is None and policy == "write_back"
+        if lazy:
+            assert len(opt._stale_host_grads) == len(opt._offload_params)
+            assert all(opt.state[p]["grad"].abs().sum() == 0 for p in opt._offload_params)
+            saved = opt.state_dict()["state"]
+            assert not opt._stale_host_grads
+            index = {id(q): i for i, q in enumerate(opt.param_groups[0]["params"])}
+            sums.append([saved[index[id(p)]]["grad"].clone() for p in opt._offload_params])
+        else:
+            sums.append([opt.state[p]["grad"].clone() for p in opt._offload_params])
         kept = [opt.device_states[p].get("grad") is not None for p in opt._offload_params]
         assert all(kept) if cache is None else not any(kept)
-    for a, b in zip(*sums):
-        assert torch.equal(a, b) and a.abs().sum() > 0
+    for a, b, c in zip(*sums):
+        assert torch.equal(a, b) and torch.equal(a, c) and a.abs().sum() > 0
+
+
+def test_grad_cache_policy_is_validated():
+    from offload_adam_amd import OffloadAdam
+
+    with pytest.raises(ValueError, match="grad_cache_policy"):
+        OffloadAdam(make_model(0), grad_cache_policy="sometimes")
 
 
 @pytest.mark.parametrize("group_params,group_bytes", [(1, 1 << 30), (3, 1 << 30), (100, 1 << 30),
@@ -889,6 +913,9 @@ def test_prefetch_budget_does_not_change_results(fixed_seed, prefetch_bytes):
                                 dict(prefetch_bytes=0), dict(grad_cache_bytes=0),
                                 dict(grad_cache_bytes=0, max_grad_norm=0.05),
                                 dict(grad_cache_bytes=40_000), dict(state_cache_bytes=0),
+                                dict(grad_cache_policy="write_through"),
+                                dict(grad_cache_policy="write_through", max_grad_norm=0.05),
+                                dict(grad_cache_policy="write_through", grad_cache_bytes=40_000),
                                 dict(state_cache_bytes=200_000, grad_cache_bytes=0),
                                 dict(state_cache_bytes=0, grad_cache_bytes=0, prefetch_bytes=0)])
 def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monkeypatch, kw):
@@ -965,7 +992,10 @@ def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monk
             for k in opt._non_grad_keys:
                 assert on_device.get((p, k)), f"kernel ran without {k} on the device"
             if opt.offload_grads and ga > 1:
-                assert on_device.get((p, "grad")), "kernel ran without the accumulated gradient"
+                # under 'write_back' a cached gradient never left the GPU
+                assert on_device.get((p, "grad")) or (
+                    p in opt._grad_cached and opt._grad_cache_write_back
+                ), "kernel ran without the accumulated gradient"
     assert set(stepped.values()) == {steps}
     # at the end of a step nothing but staged states of the next step is live, and
     # every state written by a kernel went back to the host
