@@ -222,12 +222,12 @@ class OffloadAdam(Optimizer):
             from ``2*(grad_accum-1)+4`` to ``4`` bytes per element each way in
             ``stochastic_rounding`` mode.  Results are bit-identical.
         grad_cache_bytes (int, keyword-only): with ``offload_grads=True``, HBM
-            that may keep the device copy of accumulated gradients alive after
-            they have been written back to the host.  The write-back happens as
-            in the reference (``state[p]['grad']`` on the host is always
-            current); what is saved is fetching the same bytes again for the next
-            micro-batch, or for ``step()`` on the clipping path.  Parameters are
-            admitted in optimizer order until the budget is used.  Default: a
+            that may keep the device copy of accumulated gradients alive between
+            micro-batches.  What is saved is fetching the same bytes again for
+            the next micro-batch, or for ``step()`` on the clipping path (and,
+            under ``grad_cache_policy='write_back'``, writing partial sums nobody
+            reads).  Parameters are admitted in optimizer order until the budget
+            is used.  Default: a
             tenth of the HBM that is free when the optimizer is built; ``0``
             fetches every time, like the reference.  Results are bit-identical.
         grad_cache_policy (str, keyword-only): when a gradient kept by
