@@ -204,8 +204,9 @@ def offloaded_step_8b(timeout_s=420):
     bench_e2e.py in a child process.  PCIe-inclusive; never part of ``value``."""
     import subprocess
 
-    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", "6",
-           "--warmup", "1"]
+    # 12 steps: the write-back that trails the last step (0.5 s) is timed with them
+    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", "12",
+           "--warmup", "2"]
     try:
         res = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout_s, cwd=str(ROOT))
         if res.returncode != 0:
@@ -214,7 +215,7 @@ def offloaded_step_8b(timeout_s=420):
         full = json.loads(res.stdout.strip().splitlines()[-1])
     except Exception as exc:  # a failed side measurement must not lose the main line
         return {"error": repr(exc)[:300]}
-    full["steps"], full["warmup"] = 6, 1
+    full["steps"], full["warmup"] = 12, 2
     keep = ("model", "mode", "steps", "warmup", "seq", "grad_accum", "offload_grads", "params", "step_s",
             "tokens_per_s", "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step",
             "d2h_GB_per_step", "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak",
