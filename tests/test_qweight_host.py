@@ -275,3 +275,107 @@ def test_leaf_module_scan():
 
     found = get_leaf_modules_with_params(nn.Sequential(Holder(), nn.LayerNorm(2)))
     assert [type(m).__name__ for m in found] == ["Linear", "LayerNorm"]
+
+
+# ------------------------------------------------- F.linear, copy_, partial loads
+
+
+def payload_of(qw):
+    return {k: v for k, v in qw.to_plain_state_dict().items()}
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("weight_cls,kw", FORMATS)
+def test_linear_forward_and_backward_equal_the_dequantised_layer(weight_cls, kw, device):
+    """``F.linear`` on a quantised weight (reference: int8.py:378-407 and the same
+    in the other formats) gives what a plain layer holding the dequantised weight
+    gives; the weight's gradient is a plain tensor of the full shape."""
+    import torch.nn.functional as F
+
+    torch.manual_seed(0)
+    out_f, in_f, batch = 64, 256, 8
+    dtype = torch.bfloat16 if device == "cuda" else torch.float32
+    w = (torch.randn(out_f, in_f) * 0.05).to(device=device, dtype=dtype)
+    b = (torch.randn(out_f) * 0.05).to(device=device, dtype=dtype).requires_grad_(True)
+    x = torch.randn(batch, in_f).to(device=device, dtype=dtype).requires_grad_(True)
+    qw = weight_cls.from_float(w, **kw).requires_grad_(True)
+    F.linear(x, qw, b).sum().backward()
+
+    x2 = x.detach().clone().requires_grad_(True)
+    b2 = b.detach().clone().requires_grad_(True)
+    w2 = qw.dequantize(dtype).detach().clone().requires_grad_(True)
+    y2 = F.linear(x2, w2, b2)
+    y2.sum().backward()
+    y = F.linear(x.detach(), qw.detach(), b.detach())
+    tol = dict(atol=1e-2, rtol=1e-2)
+    assert torch.allclose(y, y2, **tol)
+    assert torch.allclose(x.grad, x2.grad, **tol)
+    assert torch.allclose(b.grad, b2.grad, **tol)
+    assert torch.allclose(qw.grad.float(), w2.grad.float(), **tol)  # stored in the weight's dtype
+    assert type(qw.grad) is torch.Tensor and qw.grad.shape == (out_f, in_f)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("weight_cls,kw", FORMATS)
+def test_copy_of_a_float_tensor_re_encodes_like_a_fresh_quantisation(weight_cls, kw, device):
+    """``qw.copy_(fp32)`` - what both optimizers do with the new master - leaves the
+    payload that ``from_float`` of the same values builds, bit for bit."""
+    torch.manual_seed(0)
+    old = (torch.randn(64, 256) * 0.05).to(device=device, dtype=torch.bfloat16)
+    new = torch.randn(64, 256, dtype=torch.float32, device=device)
+    qw = weight_cls.from_float(old, **kw)
+    qw.copy_(new)
+    fresh = weight_cls.from_float(new, **kw)
+    a, b = payload_of(qw), payload_of(fresh)
+    assert a.keys() == b.keys()
+    for key in a:
+        if "quant_state" in key:
+            continue  # serialised metadata; it names the dtype the weight was built from
+        if a[key].dtype == b[key].dtype:
+            assert torch.equal(a[key], b[key]), key
+        else:  # from_float of an fp32 tensor may keep wider scales than the stored ones
+            assert torch.equal(a[key].float(), b[key].to(a[key].dtype).float()), key
+
+
+@pytest.mark.parametrize("weight_cls,kw", FORMATS)
+def test_partial_checkpoint_reports_the_keys_it_lacks(weight_cls, kw):
+    src, dst = build(weight_cls, kw, "cpu", seed=0), build(weight_cls, kw, "cpu", seed=1)
+    full = src.state_dict()
+    dropped = "l2." + weight_cls.canonical_key_suffixes()[0]
+    assert dropped in full
+    partial = {k: v for k, v in full.items() if k != dropped}
+    missing, unexpected = dst.load_state_dict(partial, strict=False)
+    assert not unexpected
+    assert missing and all(k.startswith("l2.") for k in missing)
+
+
+def test_update_hf_config_is_opt_in_and_needs_a_config():
+    from types import SimpleNamespace
+
+    model = TwoLinears().to(torch.bfloat16)
+    model.config = SimpleNamespace()
+    quantize_linears(model, Int8QWeight)  # update_hf_config defaults to False
+    assert not hasattr(model.config, "quantization_config")
+    bare = TwoLinears().to(torch.bfloat16)
+    quantize_linears(bare, Int8QWeight, update_hf_config=True)  # no .config: nothing to patch
+    assert not hasattr(bare, "config")
+
+
+def test_save_quantized_pretrained_merges_the_config(tmp_path):
+    import json
+
+    from offload_adam_amd.qweight import save_quantized_pretrained
+
+    class Saves(TwoLinears):
+        def save_pretrained(self, directory):
+            directory.mkdir(parents=True, exist_ok=True)
+            (directory / "config.json").write_text(json.dumps({"model_type": "toy"}))
+
+    model = Saves().to(torch.bfloat16)
+    quantize_linears(model, Int4QWeight, group_size=128, skip_patterns=("l2",))
+    save_quantized_pretrained(model, tmp_path / "out", Int4QWeight, skip_patterns=("l2",),
+                              group_size=128)
+    written = json.loads((tmp_path / "out" / "config.json").read_text())
+    assert written["model_type"] == "toy"
+    assert written["quantization_config"] == Int4QWeight.build_hf_quantization_config(
+        skip_patterns=("l2",), group_size=128)
