@@ -700,7 +700,11 @@ class OffloadAdam(Optimizer):
                 dev["grad"].add_(p.grad)
         elif state["host_grad_valid"]:
             kept = dev.get("grad")
-            if kept is not None and kept.dtype == p.grad.dtype and p.grad.is_contiguous():
+            # fetches the sum when it is not here, and waits for a fetch under way
+            self._ensure_on_device(p, ["grad"])
+            if kept is None:
+                dev["grad"].add_(p.grad)  # a fresh copy from the host: nobody else reads it
+            elif kept.dtype == p.grad.dtype and p.grad.is_contiguous():
                 # The device copy was kept (grad_cache_bytes) and its write-back may
                 # still be reading it.  The sum goes into this micro-batch's buffer
                 # instead (a + b == b + a bit for bit), so the compute stream never
@@ -709,11 +713,10 @@ class OffloadAdam(Optimizer):
                 p.grad.add_(kept)
                 dev["grad"] = p.grad
             else:
-                if kept is not None and p in self.d2h_events:
+                if p in self.d2h_events:
                     # in-place sum: the write-back must have read the kept copy first
                     self._compute_stream().wait_event(self.d2h_events[p])
-                self._ensure_on_device(p, ["grad"])
-                dev["grad"].add_(p.grad)
+                kept.add_(p.grad)
         else:
             dev["grad"] = p.grad
             state["host_grad_valid"] = True

@@ -1059,3 +1059,40 @@ def test_a_backward_pass_that_raises_does_not_stall_later_ones(fixed_seed):
     torch.cuda.synchronize()
     steps = {st["step"] for st in opt.state.values()}
     assert min(steps) >= 3
+
+
+@pytest.mark.parametrize("kw", [dict(grad_cache_bytes=0, state_cache_bytes=0), dict(),
+                                dict(grad_cache_policy="write_through")])
+def test_accumulation_waits_for_transfers_of_a_large_gradient(fixed_seed, kw):
+    """A 134 MB gradient sum takes over 2 ms to cross the link in either direction,
+    far longer than the kernels around it: an add that does not wait for the fetch
+    of the sum, or overwrites it under its write-back, gives different bits."""
+    from offload_adam_amd import Adam, OffloadAdam
+
+    def build():
+        torch.manual_seed(0)
+        return nn.Sequential(nn.Linear(8192, 8192, bias=False)).to(device="cuda", dtype=BF16)
+
+    g = torch.Generator().manual_seed(3)
+    data = [torch.randn(4, 8192, generator=g).to(device="cuda", dtype=BF16) for _ in range(6)]
+
+    def loss(model, x):
+        return model(x).float().pow(2).mean()
+
+    ref = build()
+    ref_opt = Adam(ref.parameters(), mode="fp31_master", lr=1e-2)
+    model = build()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, **kw)
+    for step in range(2):
+        for mb in range(3):
+            x = data[step * 3 + mb]
+            loss(ref, x).backward()
+            opt.ready_for_optimizer_step = mb == 2
+            loss(model, x).backward()
+        ref_opt.step()
+        ref_opt.zero_grad(set_to_none=True)
+        opt.step()
+    torch.cuda.synchronize()
+    assert_same_params(ref, model)
