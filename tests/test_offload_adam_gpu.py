@@ -1061,38 +1061,76 @@ def test_a_backward_pass_that_raises_does_not_stall_later_ones(fixed_seed):
     assert min(steps) >= 3
 
 
-@pytest.mark.parametrize("kw", [dict(grad_cache_bytes=0, state_cache_bytes=0), dict(),
-                                dict(grad_cache_policy="write_through")])
-def test_accumulation_waits_for_transfers_of_a_large_gradient(fixed_seed, kw):
-    """A 134 MB gradient sum takes over 2 ms to cross the link in either direction,
-    far longer than the kernels around it: an add that does not wait for the fetch
-    of the sum, or overwrites it under its write-back, gives different bits."""
+LARGE_CASES = [
+    ("fp31_master", dict(grad_cache_bytes=0, state_cache_bytes=0)),
+    ("fp31_master", dict()),
+    ("fp31_master", dict(grad_cache_policy="write_through")),
+    ("fp31_master", dict(state_cache_bytes=0)),
+    ("fp31_master", dict(prefetch_bytes=0, grad_cache_bytes=0)),
+    ("fp31_master", dict(offload_grads=False)),
+    ("fp31_master", dict(prefetch_policy="lazy", grad_cache_bytes=0)),
+    ("fp31_master", dict(max_grad_norm=1e-3)),
+    ("fp31_master", dict(max_grad_norm=1e-3, grad_cache_bytes=0, state_cache_bytes=0)),
+    ("fp31_master", dict(max_grad_norm=1e-3, grad_cache_policy="write_through")),
+    ("fp31_master", dict(max_grad_norm=1e-3, offload_grads=False)),
+    ("stochastic_rounding", dict()),
+    ("stochastic_rounding", dict(grad_cache_bytes=0, state_cache_bytes=0)),
+    ("fp32_master", dict()),
+    ("fp32_master", dict(grad_cache_bytes=0, state_cache_bytes=0)),
+]
+
+
+@pytest.mark.parametrize("mode,kw", LARGE_CASES)
+def test_large_parameters_equal_adam(fixed_seed, mode, kw):
+    """Two 134 MB weights: each of their transfers takes over 2 ms, far longer than
+    the kernels around it, so a kernel that does not wait for a fetch under way, or
+    that overwrites a buffer under its write-back, gives different bits than the
+    optimizer without offloading (tiny tensors cross the link before anything can
+    overtake them and would hide it).  Hook path and clipping path, every cache
+    setting."""
     from offload_adam_amd import Adam, OffloadAdam
+    from offload_adam_amd.grad_clip import clip_coef_, grad_norm_
 
     def build():
         torch.manual_seed(0)
-        return nn.Sequential(nn.Linear(8192, 8192, bias=False)).to(device="cuda", dtype=BF16)
+        return nn.Sequential(nn.Linear(8192, 8192, bias=False), nn.LayerNorm(8192),
+                             nn.Linear(8192, 8192, bias=False)).to(device="cuda", dtype=BF16)
 
     g = torch.Generator().manual_seed(3)
-    data = [torch.randn(4, 8192, generator=g).to(device="cuda", dtype=BF16) for _ in range(6)]
+    steps, ga = 3, 3
+    data = [torch.randn(4, 8192, generator=g).to(device="cuda", dtype=BF16)
+            for _ in range(steps * ga)]
 
     def loss(model, x):
         return model(x).float().pow(2).mean()
 
+    max_norm = kw.get("max_grad_norm")
     ref = build()
-    ref_opt = Adam(ref.parameters(), mode="fp31_master", lr=1e-2)
+    ref_opt = Adam(ref.parameters(), mode=mode, lr=1e-2)
+    ref_params = list(ref.parameters())
+    norms = torch.zeros(len(ref_params), dtype=BF16, device="cuda")
+    coef = torch.ones((), dtype=BF16, device="cuda")
     model = build()
     with warnings.catch_warnings():
         warnings.simplefilter("ignore")
-        opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, **kw)
-    for step in range(2):
-        for mb in range(3):
-            x = data[step * 3 + mb]
+        opt = OffloadAdam(model, mode=mode, lr=1e-2, **kw)
+    assert len(opt._offload_params) == 2
+    for step in range(steps):
+        for mb in range(ga):
+            x = data[step * ga + mb]
             loss(ref, x).backward()
-            opt.ready_for_optimizer_step = mb == 2
+            opt.ready_for_optimizer_step = mb == ga - 1
             loss(model, x).backward()
+        if max_norm is not None:
+            for i, p in enumerate(ref_params):
+                grad_norm_(p.grad.reshape(-1), norms[i])
+            clip_coef_(norms, max_norm, coef)
+            for p in ref_params:
+                p.grad.mul_(coef)
         ref_opt.step()
         ref_opt.zero_grad(set_to_none=True)
         opt.step()
     torch.cuda.synchronize()
+    if max_norm is not None:
+        assert float(coef) < 1.0
     assert_same_params(ref, model)
