@@ -1134,3 +1134,48 @@ def test_large_parameters_equal_adam(fixed_seed, mode, kw):
     if max_norm is not None:
         assert float(coef) < 1.0
     assert_same_params(ref, model)
+
+
+@pytest.mark.parametrize("fmt", ["int8", "int4", "nf4", "nvfp4"])
+@pytest.mark.parametrize("kw", [dict(), dict(grad_cache_bytes=0, state_cache_bytes=0)])
+def test_large_quantised_parameters_equal_adam(fmt, kw):
+    """The same with two quantised 8192 x 8192 weights (268 MB of fp32 master each):
+    payloads and masters end up bit-identical to the optimizer without offloading."""
+    from offload_adam_amd import Adam, OffloadAdam
+    from offload_adam_amd.qweight import FORMATS, QWeightBase, quantize_linears
+
+    def build():
+        torch.manual_seed(0)
+        m = nn.Sequential(nn.Linear(8192, 8192, bias=False), nn.LayerNorm(8192),
+                          nn.Linear(8192, 8192, bias=False)).to(device="cuda", dtype=BF16)
+        assert len(quantize_linears(m, FORMATS[fmt]).quantized) == 2
+        return m
+
+    g = torch.Generator().manual_seed(3)
+    data = [torch.randn(4, 8192, generator=g).to(device="cuda", dtype=BF16) for _ in range(6)]
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        ref = build()
+        ref_opt = Adam(ref.parameters(), mode="fp32_master", lr=1e-3)
+        model = build()
+        opt = OffloadAdam(model, mode="fp32_master", lr=1e-3, **kw)
+        for step in range(3):
+            for mb in range(2):
+                x = data[step * 2 + mb]
+                ref(x).float().pow(2).mean().backward()
+                opt.ready_for_optimizer_step = mb == 1
+                model(x).float().pow(2).mean().backward()
+            ref_opt.step()
+            ref_opt.zero_grad(set_to_none=True)
+            opt.step()
+    torch.cuda.synchronize()
+    for (n, pr), (_, p) in zip(ref.named_parameters(), model.named_parameters()):
+        if isinstance(p.data, QWeightBase):
+            for name in type(p.data)._PAYLOAD:
+                a, b = getattr(pr.data, name), getattr(p.data, name)
+                assert torch.equal(a.reshape(-1).view(torch.uint8),
+                                   b.reshape(-1).view(torch.uint8)), (n, name)
+            assert torch.equal(ref_opt.state[pr]["master_params"].cpu(),
+                               opt.state[p]["master_params"]), n
+        else:
+            assert torch.equal(pr.view(torch.int16), p.view(torch.int16)), n
