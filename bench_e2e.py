@@ -308,7 +308,9 @@ def run(args):
                "nf4": qweight.NF4QWeight, "nvfp4": qweight.NVFP4QWeight}[args.qat]
         report = qweight.quantize_linears(model, cls, skip_patterns=("lm_head",))
         out["qat"] = {"format": args.qat, "quantized_linears": len(report.quantized),
-                      "incompatible": len(report.incompatible)}
+                      "incompatible": len(report.incompatible),
+                      "cache_dequantized": args.cache_dequantized}
+        qweight.cache_dequantized_weights(args.cache_dequantized)
         torch.cuda.empty_cache()
         out["model_gpu_GiB"] = round(torch.cuda.memory_allocated() / 1024**3, 2)
     n_params = sum(p.numel() for p in model.parameters())
@@ -452,6 +454,9 @@ def main():
                     help="OffloadAdam(state_cache_bytes=...): HBM for optimizer states kept on the "
                          "GPU after their write-back (default: the optimizer's; 0 = none, like "
                          "the reference)")
+    ap.add_argument("--cache-dequantized", action="store_true",
+                    help="with --qat: qweight.cache_dequantized_weights(True), one decode per "
+                         "weight per step instead of one per forward / re-computation / backward")
     ap.add_argument("--grad-cache-policy", default="write_back",
                     choices=["write_back", "write_through"],
                     help="OffloadAdam(grad_cache_policy=...): 'write_through' sends every partial "

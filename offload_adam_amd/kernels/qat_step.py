@@ -21,8 +21,9 @@ def _is_pow2(v):
 
 
 def _plan(qw):
-    """(entry point, payload arguments before the stream) for a weight subclass,
-    or None when the fused kernels do not cover its layout."""
+    """(entry point, payload arguments before the stream, payload tensors the
+    kernel writes) for a weight subclass, or None when the fused kernels do not
+    cover its layout."""
     from ..qweight import Int4QWeight, Int8QWeight, NF4QWeight, NVFP4QWeight, _codec_ops
 
     rows, cols = qw.shape
@@ -61,7 +62,7 @@ def _plan(qw):
     for t in payload:
         if not t.is_cuda or not t.is_contiguous() or t.data_ptr() % 16 != 0:
             return None
-    return name, tail
+    return name, tail, payload
 
 
 def adam_step_requant(qweight, states, lr, weight_decay, beta1, beta2, eps, step,
@@ -79,7 +80,7 @@ def adam_step_requant(qweight, states, lr, weight_decay, beta1, beta2, eps, step
     plan = _plan(qweight)
     if plan is None:
         return False
-    name, tail = plan
+    name, tail, payload = plan
     for key, dtype in (("grad", torch.bfloat16), ("exp_avg", torch.bfloat16),
                        ("exp_avg_sq", torch.bfloat16), ("master_params", torch.float32)):
         _common.check_tensor(states[key], f"states['{key}']", dtype, n, dev)
@@ -96,4 +97,7 @@ def adam_step_requant(qweight, states, lr, weight_decay, beta1, beta2, eps, step
             c_float(b1h), c_float(b2h), c_float(eps), c_int(1 if decoupled_weight_decay else 0),
             _lib.ptr(clip_coef), *tail, _lib.current_stream_ptr())
     _lib.check(code, name)
+    from ..qweight._codec_ops import mark_written
+
+    mark_written(*payload)
     return True

@@ -53,6 +53,15 @@ def _call(name, device, *args):
 # -------------------------------------------------------------------- int8
 
 
+def mark_written(*tensors):
+    """The kernels write payload tensors through raw pointers, which autograd's
+    version counters do not see; bump them, as an in-place torch op would, so
+    that anything keyed on a payload's version (the dequantisation cache of the
+    linear layers) notices."""
+    for t in tensors:
+        torch.autograd.graph.increment_version(t)
+
+
 def quantize_int8_into(src, weight, scales):
     """Per-row symmetric int8 codes of ``src`` into ``weight`` (R,C) int8 and
     ``scales`` (R,) float."""
@@ -63,6 +72,7 @@ def quantize_int8_into(src, weight, scales):
     _call("oa_quant_int8", src.device, _lib.ptr(src), c_int(_lib.dtype_code(src.dtype)),
           c_int64(stride), c_int64(rows), c_int64(cols), _lib.ptr(weight), _lib.ptr(scales),
           c_int(_lib.dtype_code(scales.dtype)))
+    mark_written(weight, scales)
 
 
 def dequantize_int8(weight, scales, out_dtype=None):
@@ -89,6 +99,7 @@ def quantize_int4_into(src, group_size, qweight, scales):
     _call("oa_quant_int4", src.device, _lib.ptr(src), c_int(_lib.dtype_code(src.dtype)),
           c_int64(stride), c_int64(rows), c_int64(cols), c_int64(group_size),
           _lib.ptr(qweight), _lib.ptr(scales), c_int(_lib.dtype_code(scales.dtype)))
+    mark_written(qweight, scales)
 
 
 def dequantize_int4(qweight, scales, group_size, out_dtype=None):
@@ -115,6 +126,7 @@ def quantize_nf4_into(src, blocksize, packed, absmax):
     _call("oa_quant_nf4", src.device, _lib.ptr(src), c_int(_lib.dtype_code(src.dtype)),
           c_int64(stride), c_int64(rows), c_int64(cols), c_int64(blocksize), _lib.ptr(packed),
           _lib.ptr(absmax))
+    mark_written(packed, absmax)
 
 
 def dequantize_nf4(packed, absmax, in_f, blocksize, out_dtype):
@@ -142,6 +154,7 @@ def quantize_nvfp4_into(src, packed, block_scale_fp8, global_scale):
     _call("oa_quant_nvfp4", src.device, _lib.ptr(src), c_int(_lib.dtype_code(src.dtype)),
           c_int64(stride), c_int64(rows), c_int64(cols), _lib.ptr(packed),
           _lib.ptr(block_scale_fp8), _lib.ptr(global_scale), _lib.ptr(ws))
+    mark_written(packed, block_scale_fp8, global_scale)
 
 
 def dequantize_nvfp4(packed, block_scale_fp8, global_scale, in_f, out_dtype):

@@ -379,3 +379,102 @@ def test_save_quantized_pretrained_merges_the_config(tmp_path):
     assert written["model_type"] == "toy"
     assert written["quantization_config"] == Int4QWeight.build_hf_quantization_config(
         skip_patterns=("l2",), group_size=128)
+
+
+# ------------------------------------------------------- dequantisation cache
+
+
+@pytest.fixture
+def dequant_cache():
+    from offload_adam_amd.qweight import cache_dequantized_weights
+
+    previous = cache_dequantized_weights(True)
+    yield
+    cache_dequantized_weights(previous)
+
+
+def count_dequantize_calls(monkeypatch, weight_cls):
+    calls = []
+    real = weight_cls.dequantize
+
+    def counting(self, dtype=None):
+        calls.append(dtype)
+        return real(self, dtype)
+
+    monkeypatch.setattr(weight_cls, "dequantize", counting)
+    return calls
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("weight_cls,kw", FORMATS)
+def test_dequantised_weights_are_decoded_once_until_the_payload_changes(
+        weight_cls, kw, device, dequant_cache, monkeypatch):
+    """With ``cache_dequantized_weights(True)`` forward and backward of several
+    micro-batches share one decode; ``copy_`` of new values (what the optimizers do),
+    loading a state dict and a payload written by hand each bring a new one; outputs
+    equal those without the cache."""
+    from offload_adam_amd.qweight import cache_dequantized_weights
+
+    model = build(weight_cls, kw, device)
+    dtype = torch.bfloat16
+    torch.manual_seed(2)
+    xs = [torch.randn(4, 256).to(device=device, dtype=dtype) for _ in range(3)]
+    calls = count_dequantize_calls(monkeypatch, weight_cls)
+    outs = []
+    for x in xs:
+        y = model(x)
+        y.float().sum().backward()
+        outs.append(y.detach().clone())
+    assert len(calls) == 2  # two quantised layers, three forward and backward passes each
+    grads = [p.grad.clone() for p in model.parameters()]
+
+    cache_dequantized_weights(False)
+    model.zero_grad(set_to_none=True)
+    for x, y_cached in zip(xs, outs):
+        y = model(x)
+        y.float().sum().backward()
+        assert torch.equal(y, y_cached)
+    for p, g in zip(model.parameters(), grads):
+        assert torch.equal(p.grad, g)
+    assert len(calls) == 2 + 2 * 2 * 3
+    cache_dequantized_weights(True)
+
+    # new values through copy_: decoded again, and the output follows
+    new = torch.randn(256, 256, dtype=torch.float32, device=device) * 0.05
+    model.l1.weight.data.copy_(new)
+    before = len(calls)
+    y_new = model(xs[0])
+    assert len(calls) == before + 1 and not torch.equal(y_new, outs[0])
+    cache_dequantized_weights(False)
+    assert torch.equal(model(xs[0]), y_new)
+    cache_dequantized_weights(True)
+
+    # a state dict from another model
+    other = build(weight_cls, kw, device, seed=5)
+    model.load_state_dict(other.state_dict())
+    assert torch.equal(model(xs[1]), other(xs[1]))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("weight_cls,kw", FORMATS)
+def test_the_fused_step_invalidates_the_dequantisation_cache(weight_cls, kw, dequant_cache):
+    """The fused step + re-encode writes the payload through raw pointers; the
+    cached decode must not survive it."""
+    from offload_adam_amd.kernels import adam_step_fp32_master
+
+    torch.manual_seed(0)
+    layer = nn.Linear(256, 128, bias=False).to(device="cuda", dtype=torch.bfloat16)
+    quantize_linears(layer, weight_cls, **kw)
+    p = layer.weight
+    x = torch.randn(4, 256, device="cuda", dtype=torch.bfloat16)
+    y0 = layer(x).detach().clone()
+    versions = [getattr(p, n)._version for n in weight_cls._PAYLOAD]
+    states = {"grad": torch.randn(128, 256, device="cuda").to(torch.bfloat16),
+              "exp_avg": torch.zeros(128, 256, device="cuda", dtype=torch.bfloat16),
+              "exp_avg_sq": torch.zeros(128, 256, device="cuda", dtype=torch.bfloat16),
+              "master_params": p.data.dequantize(torch.float32).contiguous()}
+    adam_step_fp32_master(p.data, states, 0.05, 0.0, 0.9, 0.999, 1e-8, 1)
+    assert all(getattr(p, n)._version > v for n, v in zip(weight_cls._PAYLOAD, versions))
+    y1 = layer(x)
+    assert not torch.equal(y0, y1)
+    assert torch.equal(y1, x @ p.data.dequantize(torch.bfloat16).T)
