@@ -22,7 +22,7 @@
 namespace oa {
 namespace {
 
-constexpr int kT = 256;
+constexpr int kT = 256;  // 128 lanes: flat kernels within 2 %, int8 encoder 36 -> 56 us
 constexpr float kEps = 1e-12f;
 
 // ------------------------------------------------------------ element access
@@ -695,7 +695,7 @@ quant_nf4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, int
   __shared__ u32x2 lut[32];
   nf4_buckets_to_lds(lut);
   const int64_t opr = cols >> 3, total = rows * opr;
-  const int64_t tile = SRC == kSrcAdam ? xcd_tile(blockIdx.x) : blockIdx.x;
+  const int64_t tile = SRC == kSrcAdam ? xcd_tile<kCodecXcdChunk>(blockIdx.x) : blockIdx.x;
   const int64_t o0 = tile * (kT * kOct) + threadIdx.x;
   float x[kOct][8];
 #pragma unroll
@@ -856,7 +856,7 @@ nvfp4_amax_partial_kernel(const void* __restrict__ src, int64_t stride, int64_t 
   if (vec) {
     const int64_t opr = cols >> 3, total = rows * opr;
     const bool flat = stride == cols;
-    const int64_t tile = SRC == kSrcAdam ? xcd_tile(blockIdx.x) : blockIdx.x;
+    const int64_t tile = SRC == kSrcAdam ? xcd_tile<kCodecXcdChunk>(blockIdx.x) : blockIdx.x;
     int64_t o = tile * kT * kAmaxUnroll + threadIdx.x;
     for (; o < total; o += step * kAmaxUnroll) {
       float x[kAmaxUnroll][8];
@@ -1452,7 +1452,7 @@ extern "C" int oa_adam_requant_nf4(const void* grad, void* exp_avg, void* exp_av
   if (!packed || !absmax) return OA_EINVAL;
   if (!aligned_to(packed, 4) || !aligned_to(absmax, 4)) return OA_EALIGN;
   hipLaunchKernelGGL((block == 64 ? quant_nf4_kernel<kSrcAdam, 8> : quant_nf4_kernel<kSrcAdam, 0>),
-                     dim3(xcd_grid(blocks_for(rows * (cols / 8)))),
+                     dim3(xcd_grid(blocks_for(rows * (cols / 8)), kCodecXcdChunk)),
                      dim3(kT), 0, static_cast<hipStream_t>(stream), nullptr, cols, rows, cols,
                      (int)(block / 8), log2i(block / 8), static_cast<uint32_t*>(packed),
                      static_cast<float*>(absmax), kFlat, ad);
@@ -1480,8 +1480,8 @@ extern "C" int oa_adam_requant_nvfp4(const void* grad, void* exp_avg, void* exp_
   // (kAmaxMaxBlocks is one), every block writes its partial maximum
   int64_t rblocks = (octets + kT - 1) / kT;
   if (rblocks > kAmaxMaxBlocks) rblocks = kAmaxMaxBlocks;
-  rblocks = xcd_grid((uint32_t)rblocks);
-  static_assert(kAmaxMaxBlocks % (kXcds * kXcdChunk) == 0, "padded grid must fit the workspace");
+  rblocks = xcd_grid((uint32_t)rblocks, kCodecXcdChunk);
+  static_assert(kAmaxMaxBlocks % (kXcds * kCodecXcdChunk) == 0, "padded grid must fit the workspace");
   float* partial = static_cast<float*>(workspace);
   // launch 1: the AdamW step, folding |new master| into per-block maxima
   hipLaunchKernelGGL(nvfp4_amax_partial_kernel<kSrcAdam>, dim3((unsigned)rblocks), dim3(kT), 0, s,

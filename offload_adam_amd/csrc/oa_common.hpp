@@ -112,26 +112,29 @@ __device__ __forceinline__ float wave_max(float x) {
 // Workgroup -> tile.  The dispatcher deals consecutive workgroups to the 8 XCDs
 // round-robin (workgroup b runs on XCD b % 8), each with its own L2.  With
 // tile = b every XCD touches every 8th tile of every array; mapping so that an
-// XCD owns runs of OA_ADAM_XCD_CHUNK consecutive tiles gives each L2 and the
-// memory channels behind it longer sequential streams (measured on a 4-read /
-// 3-write stream kernel of this shape: +3 % at 15 GB, +10 % at 0.8 GB per
-// launch).  The map is a bijection on [0, round_up(tiles, 8 * chunk)); grids are
-// padded to that size and surplus workgroups exit.
-#ifndef OA_ADAM_XCD_CHUNK
-#define OA_ADAM_XCD_CHUNK 64
+// XCD owns runs of CHUNK consecutive tiles gives each L2 and the memory channels
+// behind it longer sequential streams (measured on a 4-read / 3-write stream
+// kernel of this shape: +3 % at 15 GB, +10 % at 0.8 GB per launch).  The map is
+// a bijection on [0, round_up(tiles, 8 * CHUNK)); grids are padded to that size
+// and surplus workgroups exit.  CHUNK is a compile-time constant of each kernel
+// family (0 = identity): the AdamW kernels and the encoders that read their
+// elements through an AdamW update have tiles of different sizes.
+#ifndef OA_CODEC_XCD_CHUNK
+#define OA_CODEC_XCD_CHUNK 64  // tiles of 2048 elements
 #endif
 constexpr uint32_t kXcds = 8;
-constexpr uint32_t kXcdChunk = OA_ADAM_XCD_CHUNK;
+constexpr uint32_t kCodecXcdChunk = OA_CODEC_XCD_CHUNK;
 
+template <uint32_t CHUNK>
 __device__ __forceinline__ uint32_t xcd_tile(uint32_t b) {
-  if (kXcdChunk == 0) return b;
+  if (CHUNK == 0) return b;
   const uint32_t x = b % kXcds, j = b / kXcds;
-  const uint32_t c = j / kXcdChunk, r = j % kXcdChunk;
-  return (c * kXcds + x) * kXcdChunk + r;
+  const uint32_t c = j / CHUNK, r = j % CHUNK;
+  return (c * kXcds + x) * CHUNK + r;
 }
-inline uint32_t xcd_grid(uint32_t tiles) {
-  if (kXcdChunk == 0) return tiles;
-  const uint32_t q = kXcds * kXcdChunk;
+inline uint32_t xcd_grid(uint32_t tiles, uint32_t chunk) {
+  if (chunk == 0) return tiles;
+  const uint32_t q = kXcds * chunk;
   return (tiles + q - 1) / q * q;
 }
 
