@@ -217,6 +217,7 @@ def offloaded_step_8b(timeout_s=420):
         return {"error": repr(exc)[:300]}
     full["steps"], full["warmup"] = 12, 2
     keep = ("model", "mode", "steps", "warmup", "seq", "grad_accum", "offload_grads", "params", "step_s",
+            "step_s_to_last_kernel",
             "tokens_per_s", "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step",
             "d2h_GB_per_step", "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak",
             "link_floor_s", "pinned_GiB", "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB", "peak_gpu_GiB", "optimizer_init_s", "copy_engines",

@@ -319,8 +319,12 @@ def run(args):
                          generator=torch.Generator(device=dev).manual_seed(i))
            for i in range(args.grad_accum)]
 
+    compute_done = {}
+
     def loop(opt, steps):
         torch.cuda.synchronize()
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        first.record()
         t0 = time.perf_counter()
         for _ in range(steps):
             for mb in range(args.grad_accum):
@@ -333,8 +337,11 @@ def run(args):
             if opt is not None:
                 opt.step()
                 opt.zero_grad()
+        last.record()  # compute stream: the write-backs still under way are on another
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / steps
+        elapsed = (time.perf_counter() - t0) / steps
+        compute_done["s"] = first.elapsed_time(last) / 1e3 / steps
+        return elapsed
 
     # 1) forward/backward only: what a step costs with a free optimizer
     loop(None, 1)
@@ -381,6 +388,9 @@ def run(args):
         timeline.close()
         out["copy_timeline"] = timeline.summary(args.steps)
     out["step_s"] = round(step_s, 4)
+    # the same steps up to the last kernel, i.e. without the write-back that trails the last
+    # step (a training run pays that once, this measurement once per `steps`)
+    out["step_s_to_last_kernel"] = round(compute_done["s"], 4)
     out["tokens_per_s"] = round(args.grad_accum * args.seq / step_s, 1)
     out["exposed_optimizer_s"] = round(step_s - out["fwd_bwd_only_s"], 4)
     out["peak_gpu_GiB"] = round(torch.cuda.max_memory_allocated() / 1024**3, 2)
