@@ -1178,3 +1178,24 @@ def test_large_quantised_parameters_equal_adam(fmt, kw):
                                opt.state[p]["master_params"]), n
         else:
             assert torch.equal(pr.view(torch.int16), p.view(torch.int16)), n
+
+
+def test_clipping_path_gives_its_default_staging_budget_to_the_state_cache():
+    """States staged ahead of step() would hold HBM through the last backward pass;
+    unless the caller sizes a budget, the optimizer keeps them instead."""
+    from offload_adam_amd import OffloadAdam
+
+    def build(**kw):
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            return OffloadAdam(make_model(0), mode="fp31_master", inplace_param_threshold=5000,
+                               **kw)
+
+    hook = build()
+    assert hook._prestage_bytes == hook._PREFETCH_BYTES > 0
+    clip = build(max_grad_norm=1.0)
+    assert clip._prestage_bytes == 0 and len(clip._state_cached) == len(clip._offload_params)
+    sized = build(max_grad_norm=1.0, prefetch_bytes=123_456)
+    assert sized._prestage_bytes == 123_456
+    sized = build(max_grad_norm=1.0, state_cache_bytes=0)
+    assert sized._prestage_bytes == sized._PREFETCH_BYTES and not sized._state_cached
