@@ -185,6 +185,23 @@ size_t oa_norm_workspace_bytes(void);
 int oa_grad_norm_bf16(const void* grad, int64_t n, void* norm_out, void* sumsq_out,
                       void* workspace, void* stream);
 
+/* oa_grad_norm_bf16 for callers that cannot allocate device memory or pass a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  No counterpart in the reference.  The partial sums live in
+ * a device array inside the library (OA_NORM_STATIC_PARTIALS floats = 64 KiB per
+ * GPU the library runs on, held until the process ends); the call allocates and
+ * frees nothing.  Same kernels and same results, bit for bit, as
+ * oa_grad_norm_bf16.  n > OA_NORM_STATIC_MAX_ELEMS returns OA_ERANGE and
+ * launches nothing.  All calls on one GPU share that GPU's array: calls that
+ * may overlap on one GPU (different streams, several threads) race on it -
+ * serialise them, or use oa_grad_norm_bf16 with one workspace per stream.  The
+ * first call on a GPU looks the array's address up (hipGetSymbolAddress): make
+ * that call outside graph capture. */
+#define OA_NORM_STATIC_PARTIALS  16384
+#define OA_NORM_STATIC_MAX_ELEMS ((int64_t)1 << 31)  /* a 4 GiB bf16 gradient */
+int oa_grad_norm_bf16_static(const void* grad, int64_t n, void* norm_out,
+                             void* sumsq_out, void* stream);
+
 /* Replaces the global-norm and clip-coefficient arithmetic of
  * OffloadAdam.step (src/offload_adam/offload_adam.py:553-561):
  *   total = vector_norm(stack(norms), 2)                        (bf16)

@@ -53,6 +53,11 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
+    # grad, n, norm_out, sumsq_out, stream
+    "oa_grad_norm_bf16_static": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
     "oa_clip_coef_bf16": (
         c_int,
         [c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p],

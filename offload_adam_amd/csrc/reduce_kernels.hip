@@ -16,9 +16,16 @@
 //
 // Clip coefficient: one small block over the bf16 norms of all parameters.
 
+#include <atomic>
+
 #include "oa_common.hpp"
 
 #pragma clang fp contract(off)
+
+// Partial sums of oa_grad_norm_bf16_static: one copy of this array per GPU,
+// held until the process ends.  In host code the name is only a handle for
+// hipGetSymbolAddress; kernels are given the address that call returns.
+static __device__ __align__(256) float scratch[OA_NORM_STATIC_PARTIALS];
 
 namespace oa {
 namespace {
@@ -152,12 +159,12 @@ using namespace oa;
 
 extern "C" size_t oa_norm_workspace_bytes(void) { return sizeof(NormWorkspace); }
 
-extern "C" int oa_grad_norm_bf16(const void* grad, int64_t n, void* norm_out,
-                                 void* sumsq_out, void* workspace, void* stream) {
-  if (n < 0 || !norm_out || !workspace || (n > 0 && !grad)) return OA_EINVAL;
-  if (!aligned_to(grad, 2) || !aligned_to(norm_out, 2) || !aligned_to(workspace, 64) ||
-      (sumsq_out && !aligned_to(sumsq_out, 4)))
-    return OA_EALIGN;
+namespace oa {
+namespace {
+
+// The two launches of a norm; `partial` holds at least kMaxBlocks floats.
+int launch_grad_norm(const void* grad, int64_t n, void* norm_out, void* sumsq_out,
+                     float* partial, hipStream_t s) {
   const uintptr_t addr = reinterpret_cast<uintptr_t>(grad);
   int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / 2);
   if (head > n) head = n;
@@ -165,8 +172,6 @@ extern "C" int oa_grad_norm_bf16(const void* grad, int64_t n, void* norm_out,
   int64_t blocks = (groups + kTileGroups - 1) / kTileGroups;
   if (blocks < 1) blocks = 1;
   if (blocks > kMaxBlocks) blocks = kMaxBlocks;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  float* partial = static_cast<NormWorkspace*>(workspace)->partial;
   hipLaunchKernelGGL(grad_norm_partial_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, s,
                      static_cast<const uint16_t*>(grad), n, (int)head, groups, partial);
   int rc = launch_status();
@@ -175,6 +180,62 @@ extern "C" int oa_grad_norm_bf16(const void* grad, int64_t n, void* norm_out,
                      (int)blocks, static_cast<uint16_t*>(norm_out),
                      static_cast<float*>(sumsq_out));
   return launch_status();
+}
+
+// Device address of `scratch` on each GPU (every GPU holds its own copy of the
+// array at its own address), looked up once per device with that device current.
+constexpr int kMaxDevices = 64;
+std::atomic<float*> g_scratch_addr[kMaxDevices];
+
+int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return static_cast<int>(err);
+  if (dev < 0 || dev >= kMaxDevices) return OA_ERANGE;
+  float* addr = g_scratch_addr[dev].load(std::memory_order_acquire);
+  if (!addr) {
+    void* sym = nullptr;
+    err = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return static_cast<int>(err);
+    if (!sym) return static_cast<int>(hipErrorInvalidSymbol);
+    addr = static_cast<float*>(sym);
+    g_scratch_addr[dev].store(addr, std::memory_order_release);  // same value from any thread
+  }
+  *out = addr;
+  return 0;
+}
+
+}  // namespace
+}  // namespace oa
+
+static_assert(OA_NORM_STATIC_PARTIALS >= kMaxBlocks, "scratch must hold every block's partial");
+static_assert(OA_NORM_STATIC_MAX_ELEMS > 0, "");
+
+extern "C" int oa_grad_norm_bf16(const void* grad, int64_t n, void* norm_out,
+                                 void* sumsq_out, void* workspace, void* stream) {
+  if (n < 0 || !norm_out || !workspace || (n > 0 && !grad)) return OA_EINVAL;
+  if (!aligned_to(grad, 2) || !aligned_to(norm_out, 2) || !aligned_to(workspace, 64) ||
+      (sumsq_out && !aligned_to(sumsq_out, 4)))
+    return OA_EALIGN;
+  return launch_grad_norm(grad, n, norm_out, sumsq_out,
+                          static_cast<NormWorkspace*>(workspace)->partial,
+                          static_cast<hipStream_t>(stream));
+}
+
+extern "C" int oa_grad_norm_bf16_static(const void* grad, int64_t n, void* norm_out,
+                                        void* sumsq_out, void* stream) {
+  if (n < 0 || !norm_out || (n > 0 && !grad)) return OA_EINVAL;
+  if (n > OA_NORM_STATIC_MAX_ELEMS) return OA_ERANGE;
+  if (!aligned_to(grad, 2) || !aligned_to(norm_out, 2) ||
+      (sumsq_out && !aligned_to(sumsq_out, 4)))
+    return OA_EALIGN;
+  float* partial = nullptr;
+  int rc = static_scratch(&partial);
+  if (rc) return rc;
+  // Every partial the second launch reads is written by the first: nothing in
+  // the array has to start at zero.
+  return launch_grad_norm(grad, n, norm_out, sumsq_out, partial,
+                          static_cast<hipStream_t>(stream));
 }
 
 extern "C" int oa_clip_coef_bf16(const void* norms, int64_t count, float max_norm,
