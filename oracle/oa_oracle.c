@@ -21,7 +21,11 @@
  *   codecs                 the reference tests' anchors (tests/test_int8.py:43-63,
  *                          tests/test_int4.py:52-69, tests/test_nf4.py:42-56,
  *                          tests/test_nvfp4.py:51-63,233-359,470-498), torch's own
- *                          float8_e4m3fn cast, an independent torch restatement
+ *                          float8_e4m3fn cast, an independent torch restatement, and
+ *                          the outputs of the reference's own pure-torch quantisers
+ *                          on its seed-0 test shapes, an outlier tensor and tie /
+ *                          threshold-edge inputs (tests/golden/codec_fixtures.npz)
+ * No function is "parity unpinned".
  */
 #include <math.h>
 #include <stdint.h>

@@ -149,3 +149,172 @@ def test_hip_fp4_anchor_boundaries_and_signed_zero():
     sat[0, 0], sat[0, 1] = 1e6, -1e6
     byte = int(NVFP4QWeight.from_float(torch.from_numpy(sat).cuda()).weight_packed[0, 0])
     assert (byte & 0xF, byte >> 4) == (7, 15)
+
+
+# ------------------------------------------------- reference-made codec fixtures
+#
+# tests/golden/codec_fixtures.npz holds inputs and the outputs of the reference's
+# pure-torch quantisers on them (written by tests/golden/make_codec_fixtures.py
+# on the CPU).  The oracle is checked against them here; the HIP kernels are
+# checked against them, through the C ABI, in the ``gpu`` test below.
+
+FIXTURES = np.load(Path(__file__).parent / "golden" / "codec_fixtures.npz")
+TORCH_DT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
+ORACLE_DT = {"bf16": "bfloat16", "fp16": "float16", "fp32": "float32"}
+
+
+def fixture_cases(fmt):
+    return sorted({k.rsplit(".", 1)[0] for k in FIXTURES.files
+                   if k.startswith(fmt + ".") and k.count(".") == 3})
+
+
+def fx(case, key):
+    return FIXTURES[f"{case}.{key}"]
+
+
+def fixture_input(case):
+    """(torch tensor in the case's dtype, the same values as fp32 numpy)."""
+    dt = TORCH_DT[case.rsplit(".", 1)[1]]
+    raw = fx(case, "x")
+    if dt == torch.float32:
+        t = torch.from_numpy(raw.view(np.float32).copy())
+    else:
+        t = torch.from_numpy(raw.view(np.int16).copy()).view(dt)
+    return t, t.float().numpy()
+
+
+def raw_bits(t):
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.float32:
+        return t.numpy().view(np.uint32)
+    if t.dtype == torch.float8_e4m3fn:
+        return t.view(torch.uint8).numpy()
+    if t.dtype in (torch.bfloat16, torch.float16):
+        return t.view(torch.int16).numpy().view(np.uint16)
+    return t.numpy()
+
+
+def cast_bits(a_f32, dt):
+    """fp32 numpy -> bits after torch's cast to ``dt``."""
+    return raw_bits(torch.from_numpy(np.ascontiguousarray(a_f32, dtype=np.float32)).to(dt))
+
+
+def test_fixture_file_covers_every_format_and_dtype():
+    for fmt, n in (("int8", 13), ("int4", 13), ("nf4", 13), ("nvfp4", 13)):
+        assert len(fixture_cases(fmt)) == n, (fmt, fixture_cases(fmt))
+    assert np.array_equal(FIXTURES["nf4.lut"].view(np.float32),
+                          np.array(GOLDEN["nf4_lut"], dtype=np.float32))
+    assert np.array_equal(FIXTURES["nvfp4.lut"].view(np.float32),
+                          np.array(GOLDEN["fp4_e2m1_lut"], dtype=np.float32))
+
+
+@pytest.mark.parametrize("case", fixture_cases("int8"))
+def test_oracle_int8_equals_reference_fixture(oracle, case):
+    t, x = fixture_input(case)
+    q, s = oracle.quant_int8(x)
+    assert np.array_equal(q, fx(case, "codes"))
+    assert np.array_equal(cast_bits(s, t.dtype), fx(case, "scales"))
+    stored = torch.from_numpy(s.copy()).to(t.dtype).float().numpy()
+    name = ORACLE_DT[case.rsplit(".", 1)[1]]
+    got = oracle.dequant_int8(q, stored, name)
+    assert np.array_equal(got.view(fx(case, "dequant").dtype), fx(case, "dequant"))
+    assert np.array_equal(oracle.dequant_int8(q, stored, "float32").view(np.uint32),
+                          fx(case, "dequant_f32"))
+
+
+@pytest.mark.parametrize("case", fixture_cases("int4"))
+def test_oracle_int4_equals_reference_fixture(oracle, case):
+    t, x = fixture_input(case)
+    group = int(fx(case, "group"))
+    qw, s = oracle.quant_int4(x, group)
+    assert np.array_equal(qw, fx(case, "qweight"))
+    assert np.array_equal(cast_bits(s, t.dtype), fx(case, "scales"))
+    # the reference's own unpacking of its words: (out_f, in_f) signed codes -8..7
+    unpacked = fx(case, "unpacked").astype(np.int64)
+    k = np.arange(x.shape[1])
+    mine = ((qw.T.astype(np.int64)[:, k // 8] >> (4 * (k % 8))) & 0xF) - 8
+    assert np.array_equal(mine, unpacked)
+    # decoding multiplies those codes by the stored scale of their group
+    stored = torch.from_numpy(s.copy()).to(t.dtype).float().numpy()
+    want = unpacked.astype(np.float32) * np.repeat(stored.T, group, axis=1)
+    assert np.array_equal(oracle.dequant_int4(qw, stored, group, "float32"), want)
+
+
+@pytest.mark.parametrize("case", fixture_cases("nf4"))
+def test_oracle_nf4_equals_reference_fixture(oracle, case):
+    t, x = fixture_input(case)
+    block = int(fx(case, "block"))
+    packed, absmax = oracle.quant_nf4(x, block)
+    assert np.array_equal(absmax.view(np.uint32), fx(case, "absmax"))
+    assert np.array_equal(packed, fx(case, "packed"))
+    assert np.array_equal(oracle.dequant_nf4(packed, absmax, block, "float32").view(np.uint32),
+                          fx(case, "dequant_f32"))
+    # 16-bit outputs are the fp32 product cast once (qweight/nf4.py:161-227)
+    want = fx(case, "dequant_f32").view(np.float32)
+    for dt, name in ((torch.bfloat16, "bfloat16"), (torch.float16, "float16")):
+        assert np.array_equal(oracle.dequant_nf4(packed, absmax, block, name), cast_bits(want, dt))
+
+
+@pytest.mark.parametrize("case", fixture_cases("nvfp4"))
+def test_oracle_nvfp4_equals_reference_fixture(oracle, case):
+    t, x = fixture_input(case)
+    packed, s8, gs = oracle.quant_nvfp4(x)
+    assert np.float32(gs).view(np.uint32) == fx(case, "global_scale")[0]
+    assert np.array_equal(s8, fx(case, "block_scale"))
+    assert np.array_equal(packed, fx(case, "packed"))
+    for short, name in ORACLE_DT.items():
+        want = fx(case, f"dequant_{short}")
+        assert np.array_equal(oracle.dequant_nvfp4(packed, s8, gs, name).view(want.dtype), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", ["int8", "int4", "nf4", "nvfp4"])
+def test_hip_codecs_equal_reference_fixtures(fmt):
+    """The eight codec kernels, through the C ABI, on the fixtures' inputs."""
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    for case in fixture_cases(fmt):
+        t, _ = fixture_input(case)
+        rows, cols = t.shape
+        src = t.cuda()
+        sdt = torch.bfloat16 if t.dtype == torch.float32 else t.dtype
+        if fmt == "int8":
+            q = torch.empty(rows, cols, dtype=torch.int8, device="cuda")
+            # the reference keeps the scales in the input's dtype (qweight/int8.py:49)
+            s = torch.empty(rows, dtype=t.dtype, device="cuda")
+            ops.quantize_int8_into(src, q, s)
+            assert np.array_equal(q.cpu().numpy(), fx(case, "codes")), case
+            assert np.array_equal(raw_bits(s), fx(case, "scales")), case
+            assert np.array_equal(raw_bits(ops.dequantize_int8(q, s, t.dtype)),
+                                  fx(case, "dequant")), case
+            assert np.array_equal(raw_bits(ops.dequantize_int8(q, s, torch.float32)),
+                                  fx(case, "dequant_f32")), case
+        elif fmt == "int4":
+            group = int(fx(case, "group"))
+            qw = torch.empty(cols // 8, rows, dtype=torch.int32, device="cuda")
+            s = torch.empty(cols // group, rows, dtype=t.dtype, device="cuda")
+            ops.quantize_int4_into(src, group, qw, s)
+            assert np.array_equal(qw.cpu().numpy(), fx(case, "qweight")), case
+            assert np.array_equal(raw_bits(s), fx(case, "scales")), case
+        elif fmt == "nf4":
+            block = int(fx(case, "block"))
+            packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+            absmax = torch.empty(rows * (cols // block), dtype=torch.float32, device="cuda")
+            ops.quantize_nf4_into(src, block, packed, absmax)
+            assert np.array_equal(raw_bits(absmax), fx(case, "absmax")), case
+            assert np.array_equal(packed.cpu().numpy(), fx(case, "packed")), case
+            assert np.array_equal(
+                raw_bits(ops.dequantize_nf4(packed, absmax, cols, block, torch.float32)),
+                fx(case, "dequant_f32")), case
+        else:
+            packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+            s8 = torch.empty(rows, cols // 16, dtype=torch.float8_e4m3fn, device="cuda")
+            gs = torch.empty((), dtype=torch.float32, device="cuda")
+            ops.quantize_nvfp4_into(src, packed, s8, gs)
+            assert raw_bits(gs.reshape(1))[0] == fx(case, "global_scale")[0], case
+            assert np.array_equal(raw_bits(s8), fx(case, "block_scale")), case
+            assert np.array_equal(packed.cpu().numpy(), fx(case, "packed")), case
+            for short, dt in TORCH_DT.items():
+                assert np.array_equal(raw_bits(ops.dequantize_nvfp4(packed, s8, gs, cols, dt)),
+                                      fx(case, f"dequant_{short}")), (case, short)
+        del sdt
