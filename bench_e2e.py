@@ -285,6 +285,105 @@ class CopyTimeline:
         }
 
 
+class StepCheck:
+    """Numerical check of one optimizer step of the 8B-style run (``--check``).
+
+    A sample of parameters (the first of every distinct shape) is followed
+    through one extra step after the timed ones: hooks registered BEFORE the
+    optimizer's capture each micro-batch's gradient, parameters and moments are
+    copied before the step, and afterwards plain fp32 torch ops on the GPU must
+    reproduce what the optimizer left behind - both moments bit for bit
+    (bf16_rne(m + (1-b1)(g-m)), bf16_rne(v + (1-b2)(g*g-v)) with g the bf16 sum
+    of the micro-batch gradients), every parameter on one of the two bf16
+    neighbours of the fp32 result (taken within 1 fp32 ulp: torch's sqrt and
+    divide are not promised correctly rounded), and the number of round-ups equal
+    to the sum of the round-up probabilities within 6 standard deviations."""
+
+    def __init__(self, torch, model):
+        self.torch, self.armed, self.grads, self.sample = torch, False, {}, {}
+        seen = set()
+        for name, p in model.named_parameters():
+            if tuple(p.shape) not in seen:
+                seen.add(tuple(p.shape))
+                self.sample[p] = name
+                p.register_post_accumulate_grad_hook(self._capture)
+
+    def _capture(self, p):
+        if self.armed and p.grad is not None:
+            self.grads.setdefault(p, []).append(p.grad.detach().clone())
+
+    def before(self, opt):
+        torch = self.torch
+        torch.cuda.synchronize()
+        self.old = {p: (p.detach().clone(), opt.state[p]["exp_avg"].to(p.device, copy=True),
+                        opt.state[p]["exp_avg_sq"].to(p.device, copy=True))
+                    for p in self.sample}
+        self.grads.clear()
+        self.armed = True
+
+    def after(self, opt, decoupled):
+        import numpy as np
+
+        if not decoupled:
+            raise SystemExit("--check covers decoupled weight decay only")
+        torch = self.torch
+        self.armed = False
+        torch.cuda.synchronize()
+        f32 = np.float32
+        group = opt.param_groups[0]
+        lr, eps, wd = float(f32(group["lr"])), float(f32(group["eps"])), group["weight_decay"]
+        lr_wd = float(f32(group["lr"]) * f32(wd))
+        beta1, beta2 = group["betas"]
+        report = {"tensors": len(self.sample), "elements": 0, "moments_exact": True,
+                  "params_on_bf16_neighbours": True, "failed": []}
+        ups = expected = variance = 0.0
+        for p, name in self.sample.items():
+            step = opt.state[p]["step"]
+            b1h = (beta1**step - beta1) / (beta1**step - 1)
+            b2h = (beta2**step - beta2) / (beta2**step - 1)
+            omb1, omb2 = float(f32(1) - f32(b1h)), float(f32(1) - f32(b2h))
+            p0, m0, v0 = (t.float() for t in self.old.pop(p))
+            total = self.grads[p][0]
+            for g in self.grads[p][1:]:
+                total.add_(g)  # bf16 += bf16, as the optimizer accumulates
+            g = total.float()
+            m = m0 + omb1 * (g - m0)
+            v = v0 + omb2 * (g * g - v0)
+            m_now = opt.state[p]["exp_avg"].to(p.device)
+            v_now = opt.state[p]["exp_avg_sq"].to(p.device)
+            if not (torch.equal(m_now, m.to(torch.bfloat16))
+                    and torch.equal(v_now, v.to(torch.bfloat16))):
+                report["moments_exact"] = False
+                report["failed"].append(name + ": moments")
+            M = p0 - lr_wd * p0
+            M = M - (lr * m) / (torch.sqrt(v) + eps)
+            mb = M.view(torch.int32)
+            pb = p.detach().view(torch.int16).to(torch.int32) << 16
+
+            def on_grid(b):
+                t = b & -0x10000
+                return (pb == t) | (pb == t + 0x10000)
+
+            ok = on_grid(mb) | on_grid(mb + 1) | on_grid(mb - 1)
+            if not bool(ok.all()):
+                report["params_on_bf16_neighbours"] = False
+                report["failed"].append(f"{name}: {int((~ok).sum())} params off the grid")
+            frac = (mb & 0xFFFF).double() / 65536.0
+            ups += float((pb != (mb & -0x10000)).double().sum())
+            expected += float(frac.sum())
+            variance += float((frac * (1 - frac)).sum())
+            report["elements"] += p.numel()
+            del p0, m0, v0, g, m, v, M, mb, pb, ok, frac
+        self.grads.clear()
+        report["round_ups"] = int(ups)
+        report["expected_round_ups"] = round(expected, 1)
+        report["round_up_sigma"] = round(variance ** 0.5, 1)
+        report["unbiased_within_6_sigma"] = abs(ups - expected) < 6.0 * variance ** 0.5 + 1e3
+        report["passed"] = (report["moments_exact"] and report["params_on_bf16_neighbours"]
+                            and report["unbiased_within_6_sigma"])
+        return report
+
+
 def run(args):
     import torch
 
@@ -318,6 +417,12 @@ def run(args):
     ids = [torch.randint(0, cfg["vocab"], (1, args.seq), device=dev,
                          generator=torch.Generator(device=dev).manual_seed(i))
            for i in range(args.grad_accum)]
+
+    check = None
+    if args.check:
+        if args.mode != "stochastic_rounding" or args.max_grad_norm is not None or args.qat:
+            raise SystemExit("--check covers the stochastic-rounding hook path (config 4)")
+        check = StepCheck(torch, model)  # its hooks must precede the optimizer's
 
     compute_done = {}
 
@@ -362,14 +467,15 @@ def run(args):
                                             else int(args.grad_cache_gib * 2**30)),
                           state_cache_bytes=(None if args.state_cache_gib is None
                                              else int(args.state_cache_gib * 2**30)),
-                          grad_cache_policy=args.grad_cache_policy)
+                          grad_cache_policy=args.grad_cache_policy, spare_hbm=args.spare_hbm)
     torch.cuda.synchronize()
     out["optimizer_init_s"] = round(time.perf_counter() - t0, 2)
     out["offloaded_params"] = len(opt._offload_params)
     out["inplace_params"] = len(opt._inplace_params)
     out["prefetch_GiB"] = round(opt._PREFETCH_BYTES / 1024**3, 2)
     out["grad_cache_GiB"] = round(sum(p.numel() for p in opt._grad_cached) * 2 / 1024**3, 2)
-    out["grad_cache_policy"] = args.grad_cache_policy
+    out["grad_cache_policy"] = "write_back" if opt._grad_cache_write_back else "write_through"
+    out["spare_hbm"] = bool(args.spare_hbm)
     out["state_cache_GiB"] = round(
         sum(p.numel() for p in opt._state_cached) * (opt._bytes_per_elem_in_flight - 2) / 1024**3, 2)
     out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
@@ -408,6 +514,10 @@ def run(args):
     st = _copy_engines.status()
     out["copy_engines"] = {k: st.get(k) for k in ("loaded", "active", "h2d_engine", "d2h_engine",
                                                   "h2d_copies", "d2h_copies", "rejected")}
+    if check is not None:
+        check.before(opt)
+        loop(opt, 1)
+        out["check"] = check.after(opt, decoupled=True)
     out["loss_finite"] = bool(math.isfinite(float(model(ids[0]))))
     return out
 
@@ -467,10 +577,18 @@ def main():
     ap.add_argument("--cache-dequantized", action="store_true",
                     help="with --qat: qweight.cache_dequantized_weights(True), one decode per "
                          "weight per step instead of one per forward / re-computation / backward")
-    ap.add_argument("--grad-cache-policy", default="write_back",
+    ap.add_argument("--grad-cache-policy", default=None,
                     choices=["write_back", "write_through"],
-                    help="OffloadAdam(grad_cache_policy=...): 'write_through' sends every partial "
-                         "gradient sum to the host after its micro-batch, like the reference")
+                    help="OffloadAdam(grad_cache_policy=...): 'write_through' (the default "
+                         "without --spare-hbm) sends every partial gradient sum to the host "
+                         "after its micro-batch, like the reference")
+    ap.add_argument("--spare-hbm", action="store_true",
+                    help="OffloadAdam(spare_hbm=True): budgets not given become a tenth of the "
+                         "free HBM each and gradients are written back lazily; without it the "
+                         "run has the reference's traffic (80.3 GB each way at 8B, ga=4)")
+    ap.add_argument("--check", action="store_true",
+                    help="after the timed steps, follow one more step numerically on a sample "
+                         "of parameters (see StepCheck); the result is in 'check'")
     ap.add_argument("--grads-on-device", action="store_true",
                     help="OffloadAdam(offload_grads=False): the gradient sum stays in HBM")
     ap.add_argument("--copy-timeline", action="store_true",

@@ -204,10 +204,21 @@ class OffloadAdam(Optimizer):
             module that owns it first in forward order (matters for parameters
             shared by several modules, e.g. tied embeddings).
         verbose (int): non-zero prints the pinned / in-place byte totals.
-        prefetch_bytes (int, keyword-only): device staging the hook path may fill
-            ahead of the gradient hooks.  Default: a tenth of the HBM that is free
-            when the optimizer is built (at least 2 GiB) - 27 GiB next to an 8B
-            model on a 288 GB MI355X, which holds most of that model's states.  The copies of a
+        spare_hbm (bool, keyword-only): ``False`` (default) reproduces the
+            reference's memory and traffic contract - nothing but a bounded
+            staging window of states lives in HBM besides the model, every
+            partial gradient sum goes back to pinned host memory after its
+            micro-batch and ``state[p]['grad']`` on the host is always current.
+            ``True`` lets the optimizer spend HBM that is free when it is built to
+            avoid crossing the host link: each of ``prefetch_bytes``,
+            ``grad_cache_bytes`` and ``state_cache_bytes`` that was not given
+            becomes ``'auto'`` (a tenth of the free HBM each) and
+            ``grad_cache_policy`` becomes ``'write_back'``.  The HBM that may be
+            held is printed once at construction.  Results are bit-identical.
+        prefetch_bytes (int | 'auto', keyword-only): device staging the hook path
+            may fill ahead of the gradient hooks.  Default 4 GiB (and never fewer
+            than the next two parameters); ``'auto'``: a tenth of the HBM that is
+            free when the optimizer is built, at least 2 GiB.  The copies of a
             parameter's states start this far ahead in backward order; once a
             step completes, the first ``prefetch_bytes`` of the next step's
             states are staged straight away and wait in HBM through the
@@ -221,34 +232,34 @@ class OffloadAdam(Optimizer):
             with ``grad_accum`` micro-batches the link traffic per step drops
             from ``2*(grad_accum-1)+4`` to ``4`` bytes per element each way in
             ``stochastic_rounding`` mode.  Results are bit-identical.
-        grad_cache_bytes (int, keyword-only): with ``offload_grads=True``, HBM
-            that may keep the device copy of accumulated gradients alive between
-            micro-batches.  What is saved is fetching the same bytes again for
-            the next micro-batch, or for ``step()`` on the clipping path (and,
+        grad_cache_bytes (int | 'auto', keyword-only): with ``offload_grads=True``,
+            HBM that may keep the device copy of accumulated gradients alive
+            between micro-batches.  What is saved is fetching the same bytes again
+            for the next micro-batch, or for ``step()`` on the clipping path (and,
             under ``grad_cache_policy='write_back'``, writing partial sums nobody
             reads).  Parameters are admitted in optimizer order until the budget
-            is used.  Default: a
-            tenth of the HBM that is free when the optimizer is built; ``0``
-            fetches every time, like the reference.  Results are bit-identical.
+            is used.  Default ``0``: fetch every time, like the reference;
+            ``'auto'``: a tenth of the HBM that is free when the optimizer is
+            built.  Results are bit-identical.
         grad_cache_policy (str, keyword-only): when a gradient kept by
-            ``grad_cache_bytes`` reaches the host.  ``'write_back'`` (default):
-            when somebody asks for it - ``state_dict()`` brings every host
-            gradient up to date before it returns - so partial sums that the next
-            micro-batch replaces anyway do not cross the link at all.
-            ``'write_through'``: after every micro-batch, as the reference does,
-            for code that reads ``optimizer.state[p]['grad']`` directly between
-            micro-batches.
-        state_cache_bytes (int, keyword-only): the same for the optimizer states:
-            HBM that may keep the device copy of a parameter's states alive
-            after the step has written them back to the host.  The host copy
-            stays current after every step; what is saved is fetching the same
-            bytes for the next step.  Parameters are admitted from the end of the
-            optimizer's order (the ones backward reaches first, whose fetch has
-            the least time to arrive).  Default: a tenth of the HBM that is free
-            when the optimizer is built (with ``max_grad_norm`` set and
+            ``grad_cache_bytes`` reaches the host.  ``'write_through'`` (default):
+            after every micro-batch, as the reference does, so
+            ``optimizer.state[p]['grad']`` is current between micro-batches.
+            ``'write_back'``: when somebody asks for it - ``state_dict()`` brings
+            every host gradient up to date before it returns - so partial sums
+            that the next micro-batch replaces anyway do not cross the link.
+        state_cache_bytes (int | 'auto', keyword-only): the same for the optimizer
+            states: HBM that may keep the device copy of a parameter's states
+            alive after the step has written them back to the host.  The host
+            copy stays current after every step; what is saved is fetching the
+            same bytes for the next step.  Parameters are admitted from the end
+            of the optimizer's order (the ones backward reaches first, whose
+            fetch has the least time to arrive).  Default ``0``: keep nothing,
+            like the reference; ``'auto'``: a tenth of the HBM that is free when
+            the optimizer is built (with ``max_grad_norm`` set and
             ``prefetch_bytes`` left alone, that budget is added: states staged
-            ahead of ``step()`` would hold the same HBM at the same time); ``0``
-            keeps nothing, like the reference.  Results are bit-identical.
+            ahead of ``step()`` would hold the same HBM at the same time).
+            Results are bit-identical.
     """
 
     supported_modes = {
@@ -270,7 +281,7 @@ class OffloadAdam(Optimizer):
     _STEP_GROUP_PARAMS = 8
     _STEP_GROUP_BYTES = 256 << 20
     _PREFETCH_MIN_PARAMS = 2  # hook path: H2D window ahead of the gradient hooks ...
-    _PREFETCH_BYTES = 8 << 30  # ... and in bytes of device staging (re-derived per instance)
+    _PREFETCH_BYTES = 4 << 30  # ... and in bytes of device staging (the default window)
 
     def __init__(
         self,
@@ -291,7 +302,8 @@ class OffloadAdam(Optimizer):
         prefetch_bytes=None,
         grad_cache_bytes=None,
         state_cache_bytes=None,
-        grad_cache_policy="write_back",
+        grad_cache_policy=None,
+        spare_hbm=False,
     ):
         if prefetch_policy not in ("eager", "lazy"):
             raise ValueError(f"prefetch_policy must be 'eager' or 'lazy' (got {prefetch_policy!r})")
@@ -305,13 +317,29 @@ class OffloadAdam(Optimizer):
         self.offload_state_keys = list(self.offload_config)
         self._non_grad_keys = [k for k in self.offload_state_keys if k != "grad"]
         self.offload_grads = bool(offload_grads)
+        # Budgets: an int, 'auto' (a tenth of the HBM free at construction) or None,
+        # which is the reference's contract unless spare_hbm asks for 'auto'.
+        for name, value in (("prefetch_bytes", prefetch_bytes),
+                            ("grad_cache_bytes", grad_cache_bytes),
+                            ("state_cache_bytes", state_cache_bytes)):
+            if value is None or value == "auto":
+                continue
+            if isinstance(value, bool) or not isinstance(value, int) or value < 0:
+                raise ValueError(f"{name} must be a non-negative int, 'auto' or None "
+                                 f"(got {value!r})")
+        self.spare_hbm = bool(spare_hbm)
+        if self.spare_hbm:
+            prefetch_bytes = "auto" if prefetch_bytes is None else prefetch_bytes
+            grad_cache_bytes = "auto" if grad_cache_bytes is None else grad_cache_bytes
+            state_cache_bytes = "auto" if state_cache_bytes is None else state_cache_bytes
+            grad_cache_policy = "write_back" if grad_cache_policy is None else grad_cache_policy
+        else:
+            grad_cache_bytes = 0 if grad_cache_bytes is None else grad_cache_bytes
+            state_cache_bytes = 0 if state_cache_bytes is None else state_cache_bytes
+            grad_cache_policy = "write_through" if grad_cache_policy is None else grad_cache_policy
         self._prefetch_bytes_arg = prefetch_bytes
-        if prefetch_bytes is not None:
-            self._PREFETCH_BYTES = int(prefetch_bytes)
-        if grad_cache_bytes is not None and grad_cache_bytes < 0:
-            raise ValueError("grad_cache_bytes must be >= 0")
-        if state_cache_bytes is not None and state_cache_bytes < 0:
-            raise ValueError("state_cache_bytes must be >= 0")
+        if isinstance(prefetch_bytes, int):
+            self._PREFETCH_BYTES = prefetch_bytes
         if grad_cache_policy not in ("write_back", "write_through"):
             raise ValueError("grad_cache_policy must be 'write_back' or 'write_through' "
                              f"(got {grad_cache_policy!r})")
@@ -365,21 +393,19 @@ class OffloadAdam(Optimizer):
         }
         self._offload_params = [p for p in params if p not in self._inplace_params]
 
-        if self._prefetch_bytes_arg is None and self._offload_params:
-            # a tenth of what is free now (the model is already on the GPU), at least 2 GiB
+        def tenth_of_free_hbm():
             dev0 = self._offload_params[0].device
-            if dev0.type == "cuda":
-                free, _ = torch.cuda.mem_get_info(dev0)
-                self._PREFETCH_BYTES = max(2 << 30, free // 10)
+            return torch.cuda.mem_get_info(dev0)[0] // 10 if dev0.type == "cuda" else 0
+
+        if self._prefetch_bytes_arg == "auto" and self._offload_params:
+            # the model is already on the GPU; at least 2 GiB
+            self._PREFETCH_BYTES = max(2 << 30, tenth_of_free_hbm())
 
         # parameters whose accumulated gradient stays on the GPU between micro-batches
         self._grad_cached = set()
         self._stale_host_grads = set()  # write_back policy: host copy older than the device's
         if self.offload_grads and self._offload_params:
-            budget = grad_cache_bytes
-            if budget is None:
-                dev0 = self._offload_params[0].device
-                budget = torch.cuda.mem_get_info(dev0)[0] // 10 if dev0.type == "cuda" else 0
+            budget = tenth_of_free_hbm() if grad_cache_bytes == "auto" else grad_cache_bytes
             for p in self._offload_params:
                 nbytes = p.numel() * 2
                 if nbytes > budget:
@@ -392,16 +418,15 @@ class OffloadAdam(Optimizer):
         # Clipping path: states staged for step() ahead of time occupy their HBM
         # through the last backward pass, when memory peaks, so keeping them instead
         # costs no more and saves the transfer (8B model: 21 GB per step, which
-        # arrived 0.1 s late beside the backward kernels).  Unless the caller sized
-        # either budget, the staging budget goes to the state cache.
-        fold = (not self._step_in_backward and prefetch_bytes is None
-                and state_cache_bytes is None)
+        # arrived 0.1 s late beside the backward kernels).  When both budgets are
+        # 'auto', the staging budget goes to the state cache.
+        fold = (not self._step_in_backward and self._prefetch_bytes_arg == "auto"
+                and state_cache_bytes == "auto" and self.spare_hbm)
         self._prestage_bytes = 0 if fold else self._PREFETCH_BYTES
         if self._offload_params:
             budget = state_cache_bytes
-            if budget is None:
-                dev0 = self._offload_params[0].device
-                budget = torch.cuda.mem_get_info(dev0)[0] // 10 if dev0.type == "cuda" else 0
+            if budget == "auto":
+                budget = tenth_of_free_hbm()
                 if fold:
                     budget += self._PREFETCH_BYTES
             per_elem = sum(torch.empty(0, dtype=d).element_size()
@@ -413,7 +438,7 @@ class OffloadAdam(Optimizer):
                 budget -= nbytes
                 self._state_cached.add(p)
 
-        if self.verbose > 0 and self._offload_params:
+        if (self.verbose > 0 or self.spare_hbm) and self._offload_params:
             cached_g = sum(p.numel() for p in self._grad_cached) * 2
             cached_s = sum(p.numel() for p in self._state_cached) * (
                 sum(torch.empty(0, dtype=d).element_size()
@@ -530,12 +555,18 @@ class OffloadAdam(Optimizer):
     def _copy_master(self, p, tensor):
         dev = self.device_states.get(p)
         if dev is not None:
-            # offloaded: let a write-back still under way land first, and forget any
-            # device copy (staged or cached) of the value being replaced
+            # offloaded: let a write-back still under way land first, and a fetch
+            # still under way finish reading the host buffer (states of the next
+            # step are staged as soon as a step completes); then forget any device
+            # copy (staged or cached) of the value being replaced
             self._flush_steps()
-            event = self.d2h_events.get(p)
-            if event is not None:
-                event.synchronize()
+            for events in (self.d2h_events, self.h2d_events):
+                event = events.get(p)
+                if event is not None:
+                    event.synchronize()
+            # every staged state of p has arrived (the event covers them all), so
+            # the ones that stay need no fence any more
+            self.h2d_events.pop(p, None)
             dev["master_params"] = None
         self.state[p]["master_params"].copy_(tensor)
 
@@ -643,6 +674,10 @@ class OffloadAdam(Optimizer):
         last = len(staged) - 1
         for i, (p, key, host, buf) in enumerate(staged):
             _copy_async(buf, host, _lib.OA_COPY_H2D, h2d)
+            # the buffer belongs to the compute stream's pool: if it is dropped
+            # before a consumer has waited for this copy, the allocator must not
+            # hand it out again while the copy still writes it
+            buf.record_stream(h2d)
             self.device_states[p][key] = buf
             if i == last or staged[i + 1][0] is not p:
                 self.h2d_events[p] = h2d.record_event()

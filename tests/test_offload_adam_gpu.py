@@ -242,9 +242,11 @@ def test_d2h_by_kernel_switch_gives_identical_results(fixed_seed, monkeypatch):
 
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("ga", [1, 3])
-def test_hook_path_equals_adam(fixed_seed, mode, ga):
+@pytest.mark.parametrize("spare_hbm", [False, True])
+def test_hook_path_equals_adam(fixed_seed, mode, ga, spare_hbm):
     ref_model, ref_opt = run_reference_adam(mode, steps=4, ga=ga, decoupled_weight_decay=True)
-    model, opt = run_offload_adam(mode, steps=4, ga=ga, decoupled_weight_decay=True)
+    model, opt = run_offload_adam(mode, steps=4, ga=ga, decoupled_weight_decay=True,
+                                  spare_hbm=spare_hbm)
     assert len(opt._offload_params) > 0 and len(opt._inplace_params) > 0
     assert_same_params(ref_model, model)
     # states agree too (host-resident vs GPU-resident)
@@ -569,7 +571,8 @@ class BranchyNet(TinyNet):
 
 
 @pytest.mark.parametrize("mode", ["fp31_master", "stochastic_rounding"])
-@pytest.mark.parametrize("kw", [dict(), dict(prefetch_bytes=0), dict(offload_grads=False)])
+@pytest.mark.parametrize("kw", [dict(), dict(spare_hbm=True), dict(prefetch_bytes=0),
+                                dict(offload_grads=False)])
 def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
     """The order of gradient hooks is learned, and prefetch runs along it; passes
     that skip modules (their hooks never fire, their prefetched states are not
@@ -608,12 +611,12 @@ def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
 
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("cache,policy", [(0, "write_back"), (40_000, "write_back"),
-                                          (40_000, "write_through"), (None, "write_back"),
-                                          (None, "write_through")])
+                                          (40_000, "write_through"), ("auto", "write_back"),
+                                          ("auto", "write_through")])
 @pytest.mark.parametrize("clip", [None, 0.05])
 def test_gradient_cache_does_not_change_results(fixed_seed, mode, cache, clip, policy):
     """grad_cache_bytes = 0 (every accumulated gradient is fetched back, as in the
-    reference), a budget that admits only some parameters, and the default, under
+    reference and by default), a budget that admits only some parameters, and 'auto', under
     either write policy: same bits as the optimizer without offloading, on the
     hook path and the clip path."""
     if clip is None:
@@ -627,18 +630,18 @@ def test_gradient_cache_does_not_change_results(fixed_seed, mode, cache, clip, p
     n_cached = len(opt._grad_cached)
     if cache == 0:
         assert n_cached == 0
-    elif cache is None:
+    elif cache == "auto":
         assert n_cached == len(opt._offload_params)
     else:
         assert 0 < n_cached < len(opt._offload_params)
 
 
 @pytest.mark.parametrize("mode", MODES)
-@pytest.mark.parametrize("cache", [0, 200_000, None])
+@pytest.mark.parametrize("cache", [0, 200_000, "auto"])
 @pytest.mark.parametrize("clip", [None, 0.05])
 def test_state_cache_does_not_change_results(fixed_seed, mode, cache, clip):
     """state_cache_bytes = 0 (every state is fetched for every step, as in the
-    reference), a budget that admits only some parameters, and the default: same
+    reference and by default), a budget that admits only some parameters, and 'auto': same
     bits; the host copies are current after every step."""
     ref_model, ref_opt = run_offload_adam(mode, steps=4, ga=2, max_grad_norm=clip,
                                           state_cache_bytes=0, grad_cache_bytes=0)
@@ -648,7 +651,7 @@ def test_state_cache_does_not_change_results(fixed_seed, mode, cache, clip):
     n_cached = len(opt._state_cached)
     if cache == 0:
         assert n_cached == 0
-    elif cache is None:
+    elif cache == "auto":
         assert n_cached == len(opt._offload_params)
     else:
         assert 0 < n_cached < len(opt._offload_params)
@@ -666,7 +669,7 @@ def test_loading_masters_replaces_cached_device_copies(fixed_seed):
     from offload_adam_amd import OffloadAdam
 
     results = []
-    for cache in (0, None):
+    for cache in (0, "auto"):
         model = make_model(0)
         with warnings.catch_warnings():
             warnings.simplefilter("ignore")
@@ -691,6 +694,52 @@ def test_loading_masters_replaces_cached_device_copies(fixed_seed):
         assert torch.equal(a, b)
 
 
+def test_loading_masters_while_the_next_step_is_prestaged(fixed_seed):
+    """Once a hook-path step completes, the states the next step touches first are
+    fetched straight away.  Loading masters at that moment must wait for that
+    fetch (it reads the host buffer about to be overwritten, and writes a device
+    buffer about to be dropped) and the next step must start from the loaded
+    values: two 134 MB masters make the fetch long enough to be under way."""
+    from offload_adam_amd import Adam, OffloadAdam
+
+    def net():
+        torch.manual_seed(0)
+        return nn.Sequential(nn.Linear(4096, 8192, bias=False), nn.GELU(),
+                             nn.Linear(8192, 4096, bias=False)).to(device="cuda", dtype=BF16)
+
+    g = torch.Generator().manual_seed(3)
+    xs = [torch.randn(8, 4096, generator=g).to(BF16).cuda() for _ in range(3)]
+    results = []
+    for offload in (False, True):
+        model = net()
+        if offload:
+            with warnings.catch_warnings():
+                warnings.simplefilter("ignore")
+                opt = OffloadAdam(model, mode="fp32_master", lr=1e-2, inplace_param_threshold=0)
+        else:
+            opt = Adam(model.parameters(), mode="fp32_master", lr=1e-2)
+        for i in range(2):
+            opt.ready_for_optimizer_step = True
+            model(xs[i]).float().square().mean().backward()
+            opt.step()
+            opt.zero_grad(set_to_none=True) if not offload else opt.zero_grad()
+        if offload:  # the next step's states are on their way
+            assert any(d.get("master_params") is not None for d in opt.device_states.values())
+        new = {n: torch.full_like(p, 0.01 * (i + 1), dtype=torch.float32)
+               for i, (n, p) in enumerate(model.named_parameters())}
+        opt.load_master_state_dict(new, model)
+        opt.ready_for_optimizer_step = True
+        model(xs[2]).float().square().mean().backward()
+        opt.step()
+        torch.cuda.synchronize()
+        results.append(([p.detach().clone() for p in model.parameters()],
+                        [opt.state[p]["master_params"].cpu().clone() for p in model.parameters()]))
+    for a, b in zip(results[0][0], results[1][0]):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for a, b in zip(results[0][1], results[1][1]):
+        assert torch.equal(a, b)
+
+
 def test_cached_gradient_reaches_the_host(fixed_seed):
     """Two micro-batches into a window, the pinned ``state['grad']`` holds the same
     sum whether or not the device copy was kept: at once under 'write_through',
@@ -699,7 +748,7 @@ def test_cached_gradient_reaches_the_host(fixed_seed):
     from offload_adam_amd import OffloadAdam
 
     sums = []
-    for cache, policy in ((0, "write_back"), (None, "write_through"), (None, "write_back")):
+    for cache, policy in ((0, "write_back"), ("auto", "write_through"), ("auto", "write_back")):
         model = make_model(0)
         with warnings.catch_warnings():
             warnings.simplefilter("ignore")
@@ -710,7 +759,7 @@ def test_cached_gradient_reaches_the_host(fixed_seed):
             opt.ready_for_optimizer_step = False
             loss_of(model, data[mb]).backward()
         torch.cuda.synchronize()
-        lazy = cache is None and policy == "write_back"
+        lazy = cache == "auto" and policy == "write_back"
         if lazy:
             assert len(opt._stale_host_grads) == len(opt._offload_params)
             assert all(opt.state[p]["grad"].abs().sum() == 0 for p in opt._offload_params)
@@ -721,9 +770,64 @@ def test_cached_gradient_reaches_the_host(fixed_seed):
         else:
             sums.append([opt.state[p]["grad"].clone() for p in opt._offload_params])
         kept = [opt.device_states[p].get("grad") is not None for p in opt._offload_params]
-        assert all(kept) if cache is None else not any(kept)
+        assert all(kept) if cache == "auto" else not any(kept)
     for a, b, c in zip(*sums):
         assert torch.equal(a, b) and torch.equal(a, c) and a.abs().sum() > 0
+
+
+def test_default_contract_is_the_reference_one(fixed_seed, capsys):
+    """Without ``spare_hbm`` nothing but the bounded staging window is kept in HBM and
+    the pinned ``state[p]['grad']`` holds the running bf16 sum after every
+    micro-batch (src/offload_adam/offload_adam.py:360-372, 513-514); with it, the HBM
+    that may be held is printed even at verbose=0 and the host gradient is current
+    in what ``state_dict()`` returns."""
+    from offload_adam_amd import OffloadAdam
+
+    def build(**kw):
+        model = make_model(0)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            return model, OffloadAdam(model, mode="stochastic_rounding", lr=1e-2,
+                                      inplace_param_threshold=5000, **kw)
+
+    model, opt = build()
+    assert capsys.readouterr().out == ""
+    assert not opt._grad_cached and not opt._state_cached and not opt._grad_cache_write_back
+    assert opt._PREFETCH_BYTES == 4 << 30 and opt._prestage_bytes == 4 << 30
+    names = {p: n for n, p in model.named_parameters()}
+    sums = {}
+
+    def capture(p):
+        g = p.grad.detach().to("cpu", copy=True)
+        sums[names[p]] = g if names[p] not in sums else sums[names[p]].add_(g)
+
+    # (hooks registered after the optimizer's would find p.grad already consumed)
+    model, sums = make_model(0), {}
+    names = {p: n for n, p in model.named_parameters()}
+    for p in model.parameters():
+        p.register_post_accumulate_grad_hook(capture)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode="stochastic_rounding", lr=1e-2, inplace_param_threshold=5000)
+    for mb, ids in enumerate(batches(3)):
+        opt.ready_for_optimizer_step = False
+        loss_of(model, ids).backward()
+        torch.cuda.synchronize()
+        for p in opt._offload_params:
+            host = opt.state[p]["grad"]
+            assert not host.is_cuda
+            assert torch.equal(host.view(torch.int16), sums[names[p]].view(torch.int16)), (mb, names[p])
+            assert opt.device_states[p].get("grad") is None  # nothing kept in HBM
+
+    model, opt = build(spare_hbm=True)
+    out = capsys.readouterr().out
+    assert "HBM the optimizer may hold" in out
+    assert opt._grad_cache_write_back and len(opt._grad_cached) == len(opt._offload_params)
+    assert len(opt._state_cached) == len(opt._offload_params)
+    with pytest.raises(ValueError, match="prefetch_bytes"):
+        build(prefetch_bytes=-1)
+    with pytest.raises(ValueError, match="state_cache_bytes"):
+        build(state_cache_bytes="lots")
 
 
 def test_grad_cache_policy_is_validated():
@@ -909,12 +1013,14 @@ def test_prefetch_budget_does_not_change_results(fixed_seed, prefetch_bytes):
 
 
 @pytest.mark.parametrize("kw", [dict(), dict(max_grad_norm=0.05), dict(offload_grads=False),
+                                dict(spare_hbm=True), dict(spare_hbm=True, max_grad_norm=0.05),
                                 dict(prefetch_bytes=0), dict(grad_cache_bytes=0),
                                 dict(grad_cache_bytes=0, max_grad_norm=0.05),
-                                dict(grad_cache_bytes=40_000), dict(state_cache_bytes=0),
-                                dict(grad_cache_policy="write_through"),
-                                dict(grad_cache_policy="write_through", max_grad_norm=0.05),
-                                dict(grad_cache_policy="write_through", grad_cache_bytes=40_000),
+                                dict(grad_cache_bytes=40_000), dict(state_cache_bytes="auto"),
+                                dict(grad_cache_bytes="auto", grad_cache_policy="write_back"),
+                                dict(spare_hbm=True, grad_cache_policy="write_through",
+                                     max_grad_norm=0.05),
+                                dict(grad_cache_policy="write_back", grad_cache_bytes=40_000),
                                 dict(state_cache_bytes=200_000, grad_cache_bytes=0),
                                 dict(state_cache_bytes=0, grad_cache_bytes=0, prefetch_bytes=0)])
 def test_transfer_issue_order_respects_the_happens_before_edges(fixed_seed, monkeypatch, kw):
@@ -1063,19 +1169,20 @@ def test_a_backward_pass_that_raises_does_not_stall_later_ones(fixed_seed):
 LARGE_CASES = [
     ("fp31_master", dict(grad_cache_bytes=0, state_cache_bytes=0)),
     ("fp31_master", dict()),
-    ("fp31_master", dict(grad_cache_policy="write_through")),
-    ("fp31_master", dict(state_cache_bytes=0)),
+    ("fp31_master", dict(spare_hbm=True)),
+    ("fp31_master", dict(spare_hbm=True, grad_cache_policy="write_through")),
+    ("fp31_master", dict(spare_hbm=True, state_cache_bytes=0)),
     ("fp31_master", dict(prefetch_bytes=0, grad_cache_bytes=0)),
     ("fp31_master", dict(offload_grads=False)),
     ("fp31_master", dict(prefetch_policy="lazy", grad_cache_bytes=0)),
     ("fp31_master", dict(max_grad_norm=1e-3)),
-    ("fp31_master", dict(max_grad_norm=1e-3, grad_cache_bytes=0, state_cache_bytes=0)),
-    ("fp31_master", dict(max_grad_norm=1e-3, grad_cache_policy="write_through")),
+    ("fp31_master", dict(max_grad_norm=1e-3, spare_hbm=True)),
+    ("fp31_master", dict(max_grad_norm=1e-3, spare_hbm=True, grad_cache_policy="write_through")),
     ("fp31_master", dict(max_grad_norm=1e-3, offload_grads=False)),
     ("stochastic_rounding", dict()),
-    ("stochastic_rounding", dict(grad_cache_bytes=0, state_cache_bytes=0)),
+    ("stochastic_rounding", dict(spare_hbm=True)),
     ("fp32_master", dict()),
-    ("fp32_master", dict(grad_cache_bytes=0, state_cache_bytes=0)),
+    ("fp32_master", dict(spare_hbm=True)),
 ]
 
 
@@ -1136,7 +1243,7 @@ def test_large_parameters_equal_adam(fixed_seed, mode, kw):
 
 
 @pytest.mark.parametrize("fmt", ["int8", "int4", "nf4", "nvfp4"])
-@pytest.mark.parametrize("kw", [dict(), dict(grad_cache_bytes=0, state_cache_bytes=0)])
+@pytest.mark.parametrize("kw", [dict(), dict(spare_hbm=True)])
 def test_large_quantised_parameters_equal_adam(fmt, kw):
     """The same with two quantised 8192 x 8192 weights (268 MB of fp32 master each):
     payloads and masters end up bit-identical to the optimizer without offloading."""
@@ -1180,9 +1287,9 @@ def test_large_quantised_parameters_equal_adam(fmt, kw):
             assert torch.equal(pr.view(torch.int16), p.view(torch.int16)), n
 
 
-def test_clipping_path_gives_its_default_staging_budget_to_the_state_cache():
+def test_clipping_path_gives_its_spare_staging_budget_to_the_state_cache():
     """States staged ahead of step() would hold HBM through the last backward pass;
-    unless the caller sizes a budget, the optimizer keeps them instead."""
+    with spare_hbm, unless the caller sizes a budget, the optimizer keeps them instead."""
     from offload_adam_amd import OffloadAdam
 
     def build(**kw):
@@ -1191,11 +1298,13 @@ def test_clipping_path_gives_its_default_staging_budget_to_the_state_cache():
             return OffloadAdam(make_model(0), mode="fp31_master", inplace_param_threshold=5000,
                                **kw)
 
-    hook = build()
+    hook = build(spare_hbm=True)
     assert hook._prestage_bytes == hook._PREFETCH_BYTES > 0
-    clip = build(max_grad_norm=1.0)
+    clip = build(max_grad_norm=1.0, spare_hbm=True)
     assert clip._prestage_bytes == 0 and len(clip._state_cached) == len(clip._offload_params)
-    sized = build(max_grad_norm=1.0, prefetch_bytes=123_456)
+    sized = build(max_grad_norm=1.0, spare_hbm=True, prefetch_bytes=123_456)
     assert sized._prestage_bytes == 123_456
-    sized = build(max_grad_norm=1.0, state_cache_bytes=0)
+    sized = build(max_grad_norm=1.0, spare_hbm=True, state_cache_bytes=0)
     assert sized._prestage_bytes == sized._PREFETCH_BYTES and not sized._state_cached
+    plain = build(max_grad_norm=1.0)
+    assert plain._prestage_bytes == plain._PREFETCH_BYTES and not plain._state_cached
