@@ -9,7 +9,20 @@ benchmark config 1: stochastic_rounding mode over the Llama-style 1.1B
 parameter set (201 tensors, 1,100,048,384 elements, 14 algorithmic bytes per
 element).  Prints ONE JSON line.
 
-Only one GPU is used; ``--gpus N`` with N > 1 exits with a message.
+After the timed region of the default workload the same line also carries
+
+* ``cpu_baseline``: benchmark config 0 exactly (fp32_master, 16,777,216
+  elements) in PyTorch eager on this host's cores;
+* ``other_configs``: config 0, the two kernel legs of config 2 (gradient norms,
+  fp31_master with the clip coefficient folded in, Llama-3-8B shapes) and the
+  codec kernels of config 3, each with its own ``roofline`` from HIP events and
+  a small ``cpu_baseline``;
+* ``offloaded_step_8b``: config 4 as a training step through ``OffloadAdam``
+  (child processes running bench_e2e.py): at the reference's traffic, with the
+  HBM caches, and the same model with the GPU-resident ``Adam``.
+
+``--only-main`` stops after the timed region.  Only one GPU is used;
+``--gpus N`` with N > 1 exits with a message.
 """
 
 import argparse
@@ -26,11 +39,12 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE counter runs of this script, each scaled by what the same counter
-# read for a 1 GiB device copy (factors 2.000 and 1.000).  Keyed by
-# (workload, launch form); the summary with the commands is
-# profiles/adam_multi_kernel_sr_c1_llama1b_hbm_traffic.txt.
-MEASURED_TRAFFIC_BYTES = {
-    ("c1_sr_llama1b", "multi_tensor"): 2_566_900_000,
+# read for a 1 GiB device copy (factors 2.000 and 1.000).  Counters cannot be
+# read from inside the run, so the figure is carried over from that profile and
+# the line says so (``traffic_source``).  Keyed by (workload, launch form).
+TRAFFIC_FROM_PROFILE = {
+    ("c1_sr_llama1b", "multi_tensor"): (
+        2_566_900_000, "profiles/adam_multi_kernel_sr_c1_llama1b_hbm_traffic.txt"),
 }
 
 BYTES_PER_ELEM = {
@@ -39,6 +53,7 @@ BYTES_PER_ELEM = {
     "fp31_master": 18,
     "fp32_master_custom_rounding": 18,
 }
+HYP = dict(lr=1e-4, wd=0.01, beta1=0.9, beta2=0.999, eps=1e-8)  # config 0's, step 10 on the CPU
 
 
 def llama_shapes(hidden, inter, layers, q_heads, kv_heads, head_dim, vocab):
@@ -108,52 +123,108 @@ def make_tensors(mode, shapes, device, seed=0):
     return out
 
 
-def cpu_baseline(mode, target_elems=256 * 1024 * 1024, iters=5):
-    """The same update math in PyTorch eager on this host's cores, on a bounded
-    sample of the workload: one flat tensor of ``target_elems`` elements (a
-    quarter of config 1), ``iters`` timed passes of about 2 s each."""
+# ------------------------------------------------------------------ CPU side
+
+
+def host_description():
+    """What the CPU figures ran on: core counts as the OS, the scheduler and
+    torch see them, CPU model, NUMA nodes."""
     import torch
 
-    from oracle import folded_betas, torch_eager
+    model = None
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for ln in fh:
+                if ln.startswith("model name"):
+                    model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        nodes = len([d for d in os.listdir("/sys/devices/system/node") if d[4:].isdigit()
+                     and d.startswith("node")])
+    except OSError:
+        nodes = None
+    try:
+        affinity = len(os.sched_getaffinity(0))
+    except AttributeError:
+        affinity = None
+    return {"os_cpu_count": os.cpu_count(), "sched_affinity": affinity,
+            "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
+            "torch_num_threads": torch.get_num_threads(), "cpu_model": model,
+            "numa_nodes": nodes}
 
-    n = target_elems
-    g = torch.Generator().manual_seed(0)
+
+def cpu_adam_inputs(mode, n, seed=0):
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
     p = (torch.randn(n, generator=g) * 0.02).to(torch.bfloat16)
     st = {
         "grad": (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16),
         "exp_avg": (torch.randn(n, generator=g) * 1e-4).to(torch.bfloat16),
         "exp_avg_sq": ((torch.randn(n, generator=g) * 1e-3) ** 2).to(torch.bfloat16),
     }
-    b1h, b2h = folded_betas(0.9, 0.999, 10)
-    args = (1e-4, 0.01, b1h, b2h, 1e-8, True)
-    if mode == "stochastic_rounding":
-        def run():
-            r = torch.randint(0, 65536, (n,), dtype=torch.int32)
-            torch_eager.adam_step_stochastic_rounding(p, st, *args, r)
-    elif mode == "fp32_master":
+    if mode == "fp32_master":
         st["master_params"] = p.float()
+    elif mode in ("fp31_master", "fp32_master_custom_rounding"):
+        st["rounding_error"] = torch.zeros(n, dtype=torch.int16)
+    return p, st
+
+
+def cpu_baseline(mode="fp32_master", n=16_777_216, budget_s=12.0, min_iters=5, clip=False):
+    """The same update math in PyTorch eager (the oracle's torch restatement, fp32
+    compute, one rounding per op) on this host's cores.  Default = benchmark
+    config 0 exactly: fp32_master, one flat tensor of 16,777,216 elements, lr 1e-4,
+    betas (0.9, 0.999), eps 1e-8, weight decay 0.01 decoupled, step 10.  Two
+    warm-up passes, then timed passes until ``budget_s`` is spent (at least
+    ``min_iters``); median and minimum reported.  Random bits of the
+    stochastic-rounding variant are drawn before the timed passes."""
+    import torch
+
+    from oracle import folded_betas, torch_eager
+
+    p, st = cpu_adam_inputs(mode, n)
+    b1h, b2h = folded_betas(HYP["beta1"], HYP["beta2"], 10)
+    args = (HYP["lr"], HYP["wd"], b1h, b2h, HYP["eps"], True)
+    coef = torch.tensor(0.3359375, dtype=torch.bfloat16) if clip else None
+    if mode == "stochastic_rounding":
+        bits = torch.randint(0, 65536, (n,), dtype=torch.int32,
+                             generator=torch.Generator().manual_seed(1))
+
+        def run():
+            torch_eager.adam_step_stochastic_rounding(p, st, *args, bits)
+    elif mode == "fp32_master":
         def run():
             torch_eager.adam_step_fp32_master(p, st, *args)
     else:
-        st["rounding_error"] = torch.zeros(n, dtype=torch.int16)
         fn = (torch_eager.adam_step_fp31_master if mode == "fp31_master"
               else torch_eager.adam_step_custom_rounding)
+
         def run():
-            fn(p, st, *args)
-    run()  # warm-up
-    times = []
-    for _ in range(iters):
+            fn(p, st, *args, clip_coef=coef)
+    run()
+    run()
+    times, spent = [], 0.0
+    while len(times) < min_iters or (spent < budget_s and len(times) < 200):
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
-    best = sorted(times)[len(times) // 2]
+        spent += times[-1]
+    med = sorted(times)[len(times) // 2]
+    alg = n * BYTES_PER_ELEM[mode]
     return {
-        "value": round(n * BYTES_PER_ELEM[mode] / best / 1e9, 3),
+        "value": round(alg / med / 1e9, 3),
         "unit": "GB/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"one flat tensor of {n} elements, {mode}, torch eager fp32 on CPU, "
-                  f"median of {iters} passes ({best:.3f} s per pass)",
+        "sample": f"{mode}{' + clip' if clip else ''}, one flat tensor of {n} elements, torch eager "
+                  f"fp32 on the host CPU, {len(times)} timed passes after 2 warm-up: median "
+                  f"{med * 1e3:.1f} ms, min {min(times) * 1e3:.1f} ms",
+        "median_ms": round(med * 1e3, 2),
+        "min_ms": round(min(times) * 1e3, 2),
+        "best_GBps": round(alg / min(times) / 1e9, 3),
+        "passes": len(times),
     }
 
 
@@ -161,7 +232,7 @@ def cpu_baselines_of_the_other_kernels(rows=512, cols=14336):
     """The C restatement (one thread) of every kernel besides the AdamW update,
     on a bounded sample: ``rows`` x ``cols`` of the codec workload's weight and as
     many elements of gradient.  GB/s of the same algorithmic bytes the GPU figures
-    of bench_kernels.py use (bf16 source and output)."""
+    use (bf16 source and output)."""
     import numpy as np
 
     import oracle
@@ -198,15 +269,238 @@ def cpu_baselines_of_the_other_kernels(rows=512, cols=14336):
             "value": out}
 
 
-def offloaded_step_8b(timeout_s=420):
-    """The second half of the metric: step time of a synthetic Llama-3-8B-shaped
-    training step through OffloadAdam (benchmark config 4), measured by
-    bench_e2e.py in a child process.  PCIe-inclusive; never part of ``value``."""
+# ------------------------------------------------------------------ GPU side
+
+
+def time_adam_workload(name, steps, warmup, *, rng=None, per_tensor=False, use_events=True,
+                       sets=1):
+    """``steps`` timed passes of the fused AdamW kernel over every tensor of
+    workload ``name`` between two device synchronisations, after ``warmup``
+    passes.  ``sets`` > 1 rotates through that many copies of the operands (one
+    per pass), so a workload smaller than the 256 MiB memory-side cache is read
+    from HBM.  Returns the figures of the bench line."""
+    import torch
+
+    from offload_adam_amd import kernels
+    from offload_adam_amd.kernels import adam_step_multi
+    from offload_adam_amd.kernels.multi import MULTI_MAX
+
+    dev = torch.device("cuda:0")
+    wl = WORKLOADS[name]
+    mode = wl["mode"]
+    operand_sets = [make_tensors(mode, wl["shapes"], dev, seed=s) for s in range(sets)]
+    tensors = operand_sets[0]
+    step_fn = getattr(kernels, "adam_step_" + mode)
+    clip = torch.tensor(0.3359375, dtype=torch.bfloat16, device=dev) if wl["clip"] else None
+    total_elems = sum(p.numel() for p, _ in tensors)
+    bytes_per_step = total_elems * BYTES_PER_ELEM[mode]
+    kw, multi_kw = {}, {}
+    if mode == "stochastic_rounding" and rng is not None:
+        kw["rng"] = rng
+        kw["seed"] = 1
+        multi_kw["rng"] = rng
+        multi_kw["seeds"] = list(range(1, len(tensors) + 1))
+
+    multi = not per_tensor
+    lists = [([p for p, _ in ts], [st for _, st in ts]) for ts in operand_sets]
+    launches_per_step = -(-len(tensors) // MULTI_MAX) if multi else len(tensors)
+
+    def one_step(step_no, events=None):
+        """One pass of the fused AdamW kernel over every tensor of the workload."""
+        which = step_no % sets
+        if multi:
+            p_list, st_list = lists[which]
+            if events is not None:
+                events[0][0].record()
+            adam_step_multi(mode, p_list, st_list, HYP["lr"], HYP["wd"], HYP["beta1"],
+                            HYP["beta2"], HYP["eps"], step_no, decoupled_weight_decay=True,
+                            clip_coef=clip, validate=False, **multi_kw)
+            if events is not None:
+                events[0][1].record()
+            return
+        for i, (p, st) in enumerate(operand_sets[which]):
+            if events is not None:
+                events[i][0].record()
+            step_fn(p, st, HYP["lr"], HYP["wd"], HYP["beta1"], HYP["beta2"], HYP["eps"], step_no,
+                    decoupled_weight_decay=True, clip_coef=clip, **kw)
+            if events is not None:
+                events[i][1].record()
+
+    for w in range(warmup):
+        one_step(w + 1)
+    torch.cuda.synchronize()
+
+    # Timed region: exactly ``steps`` steps, bracketed by device synchronisation.
+    # Events are recorded on the stream the kernels run on (torch's current
+    # stream) and read back after the closing synchronisation.
+    pairs_per_step = 1 if multi else len(tensors)
+    all_events = []
+    t0 = time.perf_counter()
+    for s in range(steps):
+        ev = None
+        if use_events:
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                  for _ in range(pairs_per_step)]
+            all_events.append(ev)
+        one_step(warmup + s + 1, ev)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms = sum(a.elapsed_time(b) for ev in all_events for a, b in ev)
+    launches = launches_per_step * len(all_events)
+
+    roofline = None
+    if use_events and launches:
+        avg_launch_s = kernel_ms / launches / 1e3
+        alg_bytes_per_launch = bytes_per_step / launches_per_step
+        achieved = alg_bytes_per_launch / avg_launch_s / 1e9
+        traffic, source = TRAFFIC_FROM_PROFILE.get(
+            (name, "multi_tensor" if multi else "per_tensor"), (None, None))
+        roofline = {
+            "bound": "hbm",
+            "kernel": f"{'adam_multi_kernel' if multi else 'adam_vec_kernel'}<{mode}>",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": traffic,
+            "traffic_source": (source + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
+                               "command; carried over, not measured in this run)") if source else None,
+            "alg_bytes_per_launch": int(alg_bytes_per_launch),
+            "avg_launch_us": round(avg_launch_s * 1e6, 2),
+            "launches": launches,
+        }
+    return {
+        "mode": mode, "tensors": len(tensors), "elements": total_elems,
+        "bytes_per_step": bytes_per_step, "elapsed_s": elapsed, "roofline": roofline,
+        "launch": "multi_tensor" if multi else "per_tensor",
+        "rng": (rng or "x8") if mode == "stochastic_rounding" else None,
+    }
+
+
+def config0_row(steps=400, warmup=20):
+    """Benchmark config 0 on the GPU: the same 335 MB of operands every step (what
+    the config describes), and rotating through six operand sets so that the
+    256 MiB memory-side cache cannot serve any of it."""
+    import torch
+
+    row = {}
+    for label, sets in (("same_operands", 1), ("rotating_6_sets", 6)):
+        r = time_adam_workload("c0_fp32_master_16m", steps, warmup, sets=sets)
+        row[label] = {"ms_per_step": round(r["elapsed_s"] / steps * 1e3, 4),
+                      "GBps_wall": round(r["bytes_per_step"] * steps / r["elapsed_s"] / 1e9, 1),
+                      "roofline": r["roofline"]}
+        torch.cuda.empty_cache()
+    row["workload"] = "fp32_master, one flat tensor of 16,777,216 elements, 20 B/elem"
+    row["floor_us_at_8TBps"] = 41.94
+    return row
+
+
+def config2_row(steps=5, warmup=2):
+    """Kernel legs of benchmark config 2 on GPU-resident buffers at the real
+    shapes (291 tensors, 8,030,261,248 elements): per-parameter gradient norms,
+    the clip coefficient, and the fp31_master step with the coefficient folded
+    into the gradient load."""
+    import torch
+
+    from offload_adam_amd import grad_clip
+
+    r = time_adam_workload("c2_fp31_clip_llama8b", steps, warmup)
+    row = {"adam_leg": {"ms_per_step": round(r["elapsed_s"] / steps * 1e3, 3),
+                        "GBps_wall": round(r["bytes_per_step"] * steps / r["elapsed_s"] / 1e9, 1),
+                        "roofline": r["roofline"], "floor_ms_at_8TBps": 18.07}}
+    torch.cuda.empty_cache()
+    # norm leg: 291 gradients scaled so that the global norm is about 3
+    dev = torch.device("cuda:0")
+    shapes = WORKLOADS["c2_fp31_clip_llama8b"]["shapes"]
+    g = torch.Generator(device=dev).manual_seed(2)
+    grads = [(torch.randn(numel(s), device=dev, generator=g) * 3.35e-5).to(torch.bfloat16)
+             for _, s in shapes]
+    slots = torch.zeros(len(grads), dtype=torch.bfloat16, device=dev)
+    coef = torch.ones((), dtype=torch.bfloat16, device=dev)
+    total = torch.zeros((), dtype=torch.bfloat16, device=dev)
+
+    def norms():
+        for i, t in enumerate(grads):
+            grad_clip.grad_norm_(t, slots[i])
+        grad_clip.clip_coef_(slots, 1.0, coef, total)
+
+    for _ in range(2):
+        norms()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 5
+    a.record()
+    for _ in range(reps):
+        norms()
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / reps
+    nbytes = 2 * sum(t.numel() for t in grads)
+    row["norm_leg"] = {
+        "ms_per_pass": round(ms, 3), "launches_per_pass": 2 * len(grads) + 1,
+        "global_norm": float(total), "clip_coef": float(coef),
+        "roofline": {"bound": "hbm", "kernel": "grad_norm_partial_kernel + grad_norm_final_kernel "
+                     "(x291) + clip_coef_kernel", "achieved": round(nbytes / ms / 1e6, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "alg_bytes_per_pass": nbytes, "traffic": None},
+        "floor_ms_at_8TBps": 2.01,
+        "note": "583 launches issued from Python: the 130 norm-sized tensors of 4096 elements "
+                "are launch-bound",
+    }
+    del grads
+    torch.cuda.empty_cache()
+    row["workload"] = ("fp31_master + clip, Llama-3-8B shapes: 291 tensors, 8,030,261,248 "
+                       "elements, norm 2 B/elem, step 18 B/elem")
+    return row
+
+
+def config3_row(reps=40):
+    """Benchmark config 3: the eight codec kernels and the fused fp32_master step
+    + re-encode on one 4096 x 14336 weight (rotating buffers), through
+    bench_kernels.py's routines."""
+    import torch
+
+    import bench_kernels
+
+    args = argparse.Namespace(reps=reps)
+    bench_kernels.SINK = rows = []
+    try:
+        bench_kernels.bench_codecs(args, torch)
+        torch.cuda.empty_cache()
+        bench_kernels.bench_qat_step(args, torch)
+    finally:
+        bench_kernels.SINK = None
+    torch.cuda.empty_cache()
+    keep = ("kernel", "alg_bytes_per_launch", "avg_launch_us", "achieved_GBps", "frac",
+            "fused_speedup")
+    return {"workload": "one 4096 x 14336 bf16 weight ~N(0, 0.02), 1 % of the entries x10",
+            "kernels": [{k: r[k] for k in keep if k in r} for r in rows]}
+
+
+def other_configs(cpu=True):
+    out = {}
+    for name, fn in (("c0_fp32_master_16m", config0_row), ("c2_fp31_clip_llama8b", config2_row),
+                     ("c3_codecs", config3_row)):
+        try:
+            out[name] = fn()
+        except Exception as exc:  # a failed side measurement must not lose the main line
+            out[name] = {"error": repr(exc)[:300]}
+    if cpu:
+        try:
+            out["c2_fp31_clip_llama8b"]["cpu_baseline"] = cpu_baseline(
+                "fp31_master", n=16_777_216, budget_s=4.0, clip=True)
+            out["c3_codecs"]["cpu_baseline"] = cpu_baselines_of_the_other_kernels()
+        except Exception as exc:
+            out["cpu_baseline_error"] = repr(exc)[:300]
+    return out
+
+
+def run_e2e(extra, steps, warmup, timeout_s):
     import subprocess
 
-    # 12 steps: the write-back that trails the last step (0.5 s) is timed with them
-    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", "12",
-           "--warmup", "2"]
+    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", str(steps),
+           "--warmup", str(warmup)] + extra
     try:
         res = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout_s, cwd=str(ROOT))
         if res.returncode != 0:
@@ -215,14 +509,41 @@ def offloaded_step_8b(timeout_s=420):
         full = json.loads(res.stdout.strip().splitlines()[-1])
     except Exception as exc:  # a failed side measurement must not lose the main line
         return {"error": repr(exc)[:300]}
-    full["steps"], full["warmup"] = 12, 2
-    keep = ("model", "mode", "steps", "warmup", "seq", "grad_accum", "offload_grads", "params", "step_s",
-            "step_s_to_last_kernel",
-            "tokens_per_s", "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step",
-            "d2h_GB_per_step", "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak",
-            "link_floor_s", "pinned_GiB", "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB", "peak_gpu_GiB", "optimizer_init_s", "copy_engines",
-            "transfer_streams")
-    return {k: full[k] for k in keep if k in full}
+    full["steps"], full["warmup"] = steps, warmup
+    keep = ("optimizer", "mode", "steps", "warmup", "seq", "grad_accum", "spare_hbm",
+            "offload_grads", "params", "step_s", "step_s_to_last_kernel", "tokens_per_s",
+            "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step", "d2h_GB_per_step",
+            "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak", "link_floor_s", "pinned_GiB",
+            "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB",
+            "peak_gpu_GiB", "optimizer_init_s", "copy_engines", "transfer_streams", "check",
+            "loss_finite")
+    row = {k: full[k] for k in keep if k in full}
+    peak = (full.get("link_peak") or {}).get("bidir_each_GBps")
+    if peak and "h2d_GBps_over_step" in full:
+        row["h2d_frac_of_bidir_peak"] = round(full["h2d_GBps_over_step"] / peak, 3)
+        row["d2h_frac_of_bidir_peak"] = round(full["d2h_GBps_over_step"] / peak, 3)
+    return row
+
+
+def offloaded_step_8b():
+    """The second half of the metric: a synthetic Llama-3-8B-shaped training step
+    (benchmark config 4: stochastic rounding, 4 micro-batches of 4096 tokens,
+    hook path), measured by bench_e2e.py in child processes.  PCIe-inclusive;
+    never part of ``value``.
+
+    * ``reference_traffic``: OffloadAdam as constructed by default - caches off,
+      every partial gradient sum written through: 80.3 GB each way per step, the
+      reference's traffic and memory contract - followed by a numerical check of
+      one more step;
+    * ``spare_hbm``: ``OffloadAdam(spare_hbm=True)``;
+    * ``resident_adam``: the same loop with the GPU-resident ``Adam`` for scale."""
+    return {
+        "model": "llama8b (32 layers, hidden 4096, vocab 128256), bf16, 1 x 4096 tokens x 4 "
+                 "micro-batches, activation checkpointing",
+        "reference_traffic": run_e2e(["--check"], steps=5, warmup=2, timeout_s=300),
+        "spare_hbm": run_e2e(["--spare-hbm"], steps=8, warmup=2, timeout_s=300),
+        "resident_adam": run_e2e(["--optimizer", "adam"], steps=4, warmup=1, timeout_s=300),
+    }
 
 
 def main():
@@ -238,13 +559,15 @@ def main():
                          "multi-tensor launch")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run three 1 GiB device copies first (reference for counter runs)")
+    ap.add_argument("--only-main", action="store_true",
+                    help="the timed region only: no CPU baseline, other configs or 8B step "
+                         "(profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-baseline-other-kernels", action="store_true",
-                    help="also time the CPU restatement of the norm and codec kernels "
-                         "(bounded sample, a few seconds) and add it to the line")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip configs 0, 2 and 3 (about half a minute)")
     ap.add_argument("--no-e2e", action="store_true",
-                    help="skip the 8B offloaded training step (bench_e2e.py, run as a child "
-                         "process after the timed region; about a minute)")
+                    help="skip the 8B training steps (bench_e2e.py, three child processes after "
+                         "the timed region; two to three minutes)")
     ap.add_argument("--no-events", action="store_true",
                     help="skip per-launch HIP events (used for profiler runs)")
     args = ap.parse_args()
@@ -256,9 +579,7 @@ def main():
 
     import torch
 
-    from offload_adam_amd import _lib, kernels
-    from offload_adam_amd.kernels import adam_step_multi
-    from offload_adam_amd.kernels.multi import MULTI_MAX
+    from offload_adam_amd import _lib
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -266,44 +587,6 @@ def main():
     _lib.load()  # fails loudly when the HIP library is not built
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-
-    wl = WORKLOADS[args.workload]
-    mode = wl["mode"]
-    tensors = make_tensors(mode, wl["shapes"], dev)
-    step_fn = getattr(kernels, "adam_step_" + mode)
-    clip = torch.tensor(0.3359375, dtype=torch.bfloat16, device=dev) if wl["clip"] else None
-    total_elems = sum(p.numel() for p, _ in tensors)
-    bytes_per_step = total_elems * BYTES_PER_ELEM[mode]
-    kw, multi_kw = {}, {}
-    if mode == "stochastic_rounding" and args.rng is not None:
-        kw["rng"] = args.rng
-        kw["seed"] = 1
-        multi_kw["rng"] = args.rng
-        multi_kw["seeds"] = list(range(1, len(tensors) + 1))
-
-    multi = not args.per_tensor
-    p_list = [p for p, _ in tensors]
-    st_list = [st for _, st in tensors]
-    launches_per_step = -(-len(tensors) // MULTI_MAX) if multi else len(tensors)
-
-    def one_step(step_no, events=None):
-        """One pass of the fused AdamW kernel over every tensor of the workload."""
-        if multi:
-            if events is not None:
-                events[0][0].record()
-            adam_step_multi(mode, p_list, st_list, 1e-4, 0.01, 0.9, 0.999, 1e-8, step_no,
-                            decoupled_weight_decay=True, clip_coef=clip, validate=False,
-                            **multi_kw)
-            if events is not None:
-                events[0][1].record()
-            return
-        for i, (p, st) in enumerate(tensors):
-            if events is not None:
-                events[i][0].record()
-            step_fn(p, st, 1e-4, 0.01, 0.9, 0.999, 1e-8, step_no,
-                    decoupled_weight_decay=True, clip_coef=clip, **kw)
-            if events is not None:
-                events[i][1].record()
 
     if args.copy_calibration:
         # A plain device copy of known size (1 GiB read + 1 GiB written), so a
@@ -315,50 +598,11 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for w in range(args.warmup):
-        one_step(w + 1)
-    torch.cuda.synchronize()
-
-    # Timed region: exactly --steps steps, bracketed by device synchronisation.
-    # Events are recorded on the stream the kernels run on (torch's current
-    # stream) and read back after the closing synchronisation.
-    use_events = not args.no_events
-    pairs_per_step = 1 if multi else len(tensors)
-    all_events = []
-    t0 = time.perf_counter()
-    for s in range(args.steps):
-        ev = None
-        if use_events:
-            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-                  for _ in range(pairs_per_step)]
-            all_events.append(ev)
-        one_step(args.warmup + s + 1, ev)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    kernel_ms = sum(a.elapsed_time(b) for ev in all_events for a, b in ev)
-    launches = launches_per_step * len(all_events)
-
-    ms_per_step = elapsed / args.steps * 1e3
-    value = bytes_per_step * args.steps / elapsed / 1e9
-
-    roofline = None
-    if use_events and launches:
-        avg_launch_s = kernel_ms / launches / 1e3
-        alg_bytes_per_launch = bytes_per_step / launches_per_step
-        achieved = alg_bytes_per_launch / avg_launch_s / 1e9
-        roofline = {
-            "bound": "hbm",
-            "kernel": f"{'adam_multi_kernel' if multi else 'adam_vec_kernel'}<{mode}>",
-            "achieved": round(achieved, 1),
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(
-                (args.workload, "multi_tensor" if multi else "per_tensor")),
-            "alg_bytes_per_launch": int(alg_bytes_per_launch),
-            "avg_launch_us": round(avg_launch_s * 1e6, 2),
-            "launches": launches,
-        }
+    r = time_adam_workload(args.workload, args.steps, args.warmup, rng=args.rng,
+                           per_tensor=args.per_tensor, use_events=not args.no_events)
+    torch.cuda.empty_cache()
+    ms_per_step = r["elapsed_s"] / args.steps * 1e3
+    value = r["bytes_per_step"] * args.steps / r["elapsed_s"] / 1e9
 
     out = {
         "metric": "fused Adam GB/s & % HBM peak; 8B offloaded step time (s), 1 GPU",
@@ -375,25 +619,29 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": args.workload,
-            "mode": mode,
-            "tensors": len(tensors),
-            "elements": total_elems,
-            "alg_bytes_per_elem": BYTES_PER_ELEM[mode],
+            "mode": r["mode"],
+            "tensors": r["tensors"],
+            "elements": r["elements"],
+            "alg_bytes_per_elem": BYTES_PER_ELEM[r["mode"]],
             "resident": "HBM",
-            "launch": "multi_tensor" if multi else "per_tensor",
-            "rng": kw.get("rng", "x8") if mode == "stochastic_rounding" else None,
+            "launch": r["launch"],
+            "rng": r["rng"],
         },
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-        "roofline": roofline,
+        "roofline": r["roofline"],
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(mode)
-    if args.cpu_baseline_other_kernels:
-        out["cpu_baseline_other_kernels"] = cpu_baselines_of_the_other_kernels()
-    if not args.no_e2e and args.workload == "c1_sr_llama1b":
-        del tensors, p_list, st_list
-        torch.cuda.empty_cache()
-        out["offloaded_step_8b"] = offloaded_step_8b()
+    side = not args.only_main
+    if side and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"]["host"] = host_description()
+        if args.workload == "c1_sr_llama1b":
+            out["cpu_baseline_c1_sample"] = cpu_baseline("stochastic_rounding", n=64 << 20,
+                                                         budget_s=4.0, min_iters=3)
+    if side and args.workload == "c1_sr_llama1b":
+        if not args.no_other_configs:
+            out["other_configs"] = other_configs(cpu=not args.no_cpu_baseline)
+        if not args.no_e2e:
+            out["offloaded_step_8b"] = offloaded_step_8b()
     print(json.dumps(out))
 
 

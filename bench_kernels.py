@@ -49,13 +49,19 @@ def timed(fn, reps, torch):
     return a.elapsed_time(b) / reps * 1e3
 
 
+SINK = None  # a list here collects the lines instead of printing them (bench.py does that)
+
+
 def line(kernel, workload, alg_bytes, us, **extra):
     gbs = alg_bytes / us / 1e3
     out = {"kernel": kernel, "workload": workload, "alg_bytes_per_launch": int(alg_bytes),
            "avg_launch_us": round(us, 2), "achieved_GBps": round(gbs, 1),
            "peak_GBps": HBM_PEAK_GBS, "frac": round(gbs / HBM_PEAK_GBS, 4), "bound": "hbm"}
     out.update(extra)
-    print(json.dumps(out), flush=True)
+    if SINK is not None:
+        SINK.append(out)
+    else:
+        print(json.dumps(out), flush=True)
 
 
 def outlier_weight(torch, seed, dtype):
