@@ -349,6 +349,13 @@ int oa_pinned_alloc(size_t bytes, int numa_node, void** out, int* os_errno);
  * pinned_alloc.py:222-232). */
 int oa_pinned_free(void* ptr);
 
+/* Pre-flight of a large request (the reference discovers a refusal only inside
+ * pinned_alloc._alloc, src/offload_adam/pinned_alloc.py:204-221, one mapping at a
+ * time): 0 when the runtime would grant `bytes` of page-locked memory right now,
+ * else the hipError_t it gives.  The block is released before returning and is
+ * never written, so the call costs no page faults and no zero-fill. */
+int oa_pinned_probe(size_t bytes);
+
 /* Replaces pinned_alloc.gpu_numa_node (src/offload_adam/pinned_alloc.py:113-128):
  * NUMA node of the PCI device behind HIP device `device`, -1 when the kernel
  * reports none. */

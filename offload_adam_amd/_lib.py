@@ -122,6 +122,7 @@ SIGNATURES = {
         [c_size_t, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int)],
     ),
     "oa_pinned_free": (c_int, [c_void_p]),
+    "oa_pinned_probe": (c_int, [c_size_t]),
     "oa_gpu_numa_node": (c_int, [c_int, ctypes.POINTER(c_int)]),
     "oa_memcpy_async": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "oa_copy_kernel_async": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),

@@ -97,6 +97,18 @@ extern "C" int oa_pinned_alloc(size_t bytes, int numa_node, void** out, int* os_
   return 0;
 }
 
+extern "C" int oa_pinned_probe(size_t bytes) {
+  size_t size = (bytes + kPage - 1) / kPage * kPage;
+  if (size == 0) size = kPage;
+  void* p = nullptr;
+  hipError_t err = hipHostMalloc(&p, size, hipHostMallocDefault);
+  if (err != hipSuccess) {
+    (void)hipGetLastError();
+    return static_cast<int>(err);
+  }
+  return static_cast<int>(hipHostFree(p));
+}
+
 extern "C" int oa_pinned_free(void* ptr) {
   if (!ptr) return 0;
   return static_cast<int>(hipHostFree(ptr));

@@ -33,7 +33,8 @@ from . import _copy_engines, _lib, _trace, grad_clip
 from ._pretrained import stream_master_from_pretrained
 from .adam import _LOSSY_MASTER_HINT, MODE_TABLE
 from .kernels import adam_step_multi
-from .pinned_alloc import numa_node_free_bytes, resolve_numa_target, zeros_pinned
+from .pinned_alloc import (alloc_pinned_states, numa_node_free_bytes, resolve_numa_target,
+                           zeros_pinned)
 from .qweight.base import QWeightBase
 
 _BF16 = torch.bfloat16
@@ -571,11 +572,16 @@ class OffloadAdam(Optimizer):
         self.state[p]["master_params"].copy_(tensor)
 
     def _alloc_pinned_states(self, params, numa_node):
+        # Every state of every parameter, carved out of a few large pinned arenas; the
+        # arenas are all obtained (or the request refused as a whole) before any
+        # value is written.
+        requests = [(p.shape, dtype) for p in params for dtype in self._host_config.values()]
+        tensors = iter(alloc_pinned_states(requests, numa_node=numa_node))
         total = 0
         for p in params:
             state = self.state[p]
-            for name, dtype in self._host_config.items():
-                t = zeros_pinned(p.shape, dtype, numa_node=numa_node)
+            for name in self._host_config:
+                t = next(tensors)
                 if name == "master_params":
                     t.copy_(p.data)  # widens bf16 losslessly; dequantises a quantised weight
                 state[name] = t

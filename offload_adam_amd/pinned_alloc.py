@@ -7,6 +7,12 @@ runtime through the library's ``oa_pinned_alloc`` (hipHostMalloc, rounded to
 4 KiB pages - no power-of-two rounding as in torch's pinned allocator), bound
 softly to a NUMA node with the thread memory policy, zero-filled by several
 threads, and released when the last tensor that views it is collected.
+
+``PinnedArena`` / ``alloc_pinned_states`` are this package's own: the optimizer
+states of a model are carved out of a few large allocations (on 4 KiB
+boundaries) instead of one runtime allocation per state, after a pre-flight
+that fails before any memory is touched when the runtime will not grant the
+total.
 """
 
 import ctypes
@@ -135,3 +141,101 @@ def zeros_pinned(shape, dtype, numa_node="auto"):
     except BaseException:
         cleanup()
         raise
+
+
+# ------------------------------------------------------------------ arenas
+
+ARENA_BYTES = 8 << 30  # a state larger than this gets an arena of its own
+
+
+def _round_up_page(nbytes):
+    return max(_PAGE_SIZE, (nbytes + _PAGE_SIZE - 1) // _PAGE_SIZE * _PAGE_SIZE)
+
+
+class PinnedArena:
+    """One page-locked, zero-filled allocation handed out in 4 KiB-aligned
+    pieces.  The pieces are views of one storage: the memory is released when
+    the arena and every tensor carved from it are gone."""
+
+    def __init__(self, nbytes, numa_node="auto"):
+        self.nbytes = _round_up_page(nbytes)
+        self._flat = zeros_pinned((self.nbytes,), torch.uint8, numa_node=numa_node)
+        self._used = 0
+
+    @property
+    def free_bytes(self):
+        return self.nbytes - self._used
+
+    def take(self, shape, dtype):
+        shape = torch.Size(shape)
+        nbytes = shape.numel() * torch.empty(0, dtype=dtype).element_size()
+        if _round_up_page(nbytes) > self.free_bytes:
+            raise ValueError("arena exhausted")
+        piece = self._flat[self._used:self._used + nbytes]
+        self._used += _round_up_page(nbytes)
+        return piece.view(dtype).view(shape)
+
+
+def largest_grantable_bytes(upper):
+    """Largest single page-locked allocation the runtime grants right now, up to
+    ``upper`` bytes, to 256 MiB (bisection over allocate-and-release probes that
+    touch no page)."""
+    lib = _lib.load()
+    step = 256 << 20
+    lo, hi = 0, max(1, -(-upper // step))
+    if lib.oa_pinned_probe(ctypes.c_size_t(hi * step)) == 0:
+        return hi * step
+    while hi - lo > 1:
+        mid = (lo + hi) // 2
+        if lib.oa_pinned_probe(ctypes.c_size_t(mid * step)) == 0:
+            lo = mid
+        else:
+            hi = mid
+    return lo * step
+
+
+def alloc_pinned_states(requests, numa_node="auto", arena_bytes=None):
+    """Zero-filled pinned tensors for ``requests`` = [(shape, dtype), ...], carved
+    from as few arenas of ``arena_bytes`` as hold them (in order, 4 KiB-aligned).
+
+    The arenas are allocated first, all of them, before any caller data moves:
+    when the runtime refuses one, those already obtained are released and a
+    ``RuntimeError`` names the total that was asked for, how much had been
+    granted, and the largest single allocation the runtime would still grant."""
+    arena_bytes = ARENA_BYTES if arena_bytes is None else int(arena_bytes)
+    sizes = [_round_up_page(torch.Size(shape).numel() * torch.empty(0, dtype=dtype).element_size())
+             for shape, dtype in requests]
+    plan, current = [], 0  # arena sizes, filled in request order
+    for size in sizes:
+        if plan and current + size <= plan[-1]:
+            current += size
+            continue
+        if plan:
+            plan[-1] = current  # close the arena at what it holds
+        plan.append(max(arena_bytes, size))
+        current = size
+    if plan:
+        plan[-1] = current
+    total = sum(plan)
+    arenas = []
+    try:
+        for nbytes in plan:
+            arenas.append(PinnedArena(nbytes, numa_node))
+    except RuntimeError as exc:
+        granted = sum(a.nbytes for a in arenas)
+        arenas.clear()
+        still = largest_grantable_bytes(total)
+        raise RuntimeError(
+            f"pinned host memory: {total / 2**30:.1f} GiB were asked for in {len(plan)} "
+            f"allocations and the runtime refused after {granted / 2**30:.1f} GiB ({exc}); the "
+            f"largest single allocation it grants now is {still / 2**30:.1f} GiB. Nothing was "
+            "kept. Page-locked memory is limited per process by the GPU driver, not by free "
+            "RAM: offload fewer bytes per element (another mode, offload_grads=False) or raise "
+            "inplace_param_threshold."
+        ) from None
+    out, index = [], 0
+    for (shape, dtype), size in zip(requests, sizes):
+        if size > arenas[index].free_bytes:
+            index += 1  # the plan above closed this arena at exactly what it holds
+        out.append(arenas[index].take(shape, dtype))
+    return out

@@ -172,6 +172,114 @@ def test_pinned_memory_is_released():
         lib.oa_pinned_free = real
 
 
+def test_states_are_carved_from_arenas_and_released_together():
+    """States come out of a few large pinned allocations on 4 KiB boundaries, in
+    request order, zero-filled and of the exact shape and dtype; an arena goes back
+    to the runtime when its last piece dies."""
+    from offload_adam_amd import _lib, pinned_alloc
+
+    lib = _lib.load()
+    real_alloc, real_free = lib.oa_pinned_alloc, lib.oa_pinned_free
+    calls, freed = [], []
+
+    def spy_alloc(size, *rest):
+        calls.append(size.value if hasattr(size, "value") else size)
+        return real_alloc(size, *rest)
+
+    def spy_free(ptr):
+        freed.append(ptr.value if hasattr(ptr, "value") else ptr)
+        return real_free(ptr)
+
+    requests = [((300, 70), BF16), ((5000,), torch.float32), ((1,), torch.int16),
+                ((40_000,), BF16), ((0,), BF16), ((33_000,), torch.float32)]
+    gc.collect()
+    lib.oa_pinned_alloc, lib.oa_pinned_free = spy_alloc, spy_free
+    try:
+        pieces = pinned_alloc.alloc_pinned_states(requests, numa_node=None, arena_bytes=128 << 10)
+        # 45056 + 20480 + 4096 | 81920 + 4096 | 135168 (its own arena): three allocations
+        assert calls == [69632, 86016, 135168]
+        for (shape, dtype), t in zip(requests, pieces):
+            assert t.shape == torch.Size(shape) and t.dtype == dtype and t.is_contiguous()
+            assert t.data_ptr() % 4096 == 0 and not t.any()
+            assert t.numel() == 0 or t.is_pinned()
+        bases = [pieces[0].data_ptr(), pieces[3].data_ptr(), pieces[5].data_ptr()]
+        assert pieces[1].data_ptr() == bases[0] + 45056
+        assert pieces[2].data_ptr() == bases[0] + 45056 + 20480
+        for t in pieces:
+            t.fill_(1)  # writable, and no piece overlaps another
+        assert all(int(t.double().sum()) == t.numel() for t in pieces)
+        keep = pieces[1]
+        del pieces, t
+        gc.collect()
+        assert set(freed) == {bases[1], bases[2]}  # the first arena still has a live piece
+        assert int(keep.double().sum()) == 5000
+        del keep
+        gc.collect()
+        assert sorted(freed) == sorted(bases)
+    finally:
+        lib.oa_pinned_alloc, lib.oa_pinned_free = real_alloc, real_free
+
+
+def test_a_request_the_runtime_cannot_grant_fails_before_anything_is_kept():
+    """The reference meets a refusal one mapping at a time, mid-construction
+    (src/offload_adam/pinned_alloc.py:204-221).  Here the arenas are obtained first:
+    a refusal releases them all and reports the total, what had been granted and the
+    largest block the runtime would still give."""
+    from offload_adam_amd import pinned_alloc
+
+    with pytest.raises(RuntimeError) as info:
+        pinned_alloc.alloc_pinned_states([((1 << 40,), torch.uint8)] * 64, numa_node=None)
+    text = str(info.value)
+    assert "65536.0 GiB were asked for in 64 allocations" in text
+    assert "refused after 0.0 GiB" in text and "largest single allocation" in text
+    # the probe behind that figure: grants are granted, refusals refused, nothing is left over
+    lib = pinned_alloc._lib.load()
+    assert lib.oa_pinned_probe(1 << 20) == 0
+    assert lib.oa_pinned_probe(1 << 46) != 0
+    t = pinned_alloc.zeros_pinned((1 << 20,), torch.uint8, numa_node=None)  # still works
+    assert t.is_pinned() and not t.any()
+
+
+def test_numa_preference_is_applied_and_the_thread_policy_restored():
+    """numa_node=k: the allocation runs under MPOL_PREFERRED(k) and the calling
+    thread is back on the default policy afterwards.  Where the kernel tells on
+    which node the pages of the mapping sit (/proc/self/numa_maps ``N<k>=`` counts,
+    or move_pages(2) with a NULL node list), they must sit on node k; a page-locked
+    block that is a mapping of the GPU's device file exposes neither, which the test
+    then states instead."""
+    import ctypes
+    import re
+
+    from offload_adam_amd.pinned_alloc import numa_node_free_bytes, zeros_pinned
+
+    if numa_node_free_bytes(0) is None:
+        pytest.skip("this host exposes no NUMA nodes")
+    libc = ctypes.CDLL(None, use_errno=True)
+    SYS_get_mempolicy, SYS_move_pages = 239, 279  # x86-64
+    node = 0
+    t = zeros_pinned((8 << 20,), torch.uint8, numa_node=node)
+    mode = ctypes.c_int(-1)
+    assert libc.syscall(SYS_get_mempolicy, ctypes.byref(mode), None, 0, None, 0) == 0
+    assert mode.value == 0  # MPOL_DEFAULT again
+    t[::4096] = 1  # the CPU has touched every page
+    n = 64
+    pages = (ctypes.c_void_p * n)(*[t.data_ptr() + i * 32 * 4096 for i in range(n)])
+    status = (ctypes.c_int * n)(*([-99] * n))
+    rc = libc.syscall(SYS_move_pages, 0, ctypes.c_ulong(n), pages, None, status, 0)
+    assert rc == 0
+    placed = [s for s in status if s >= 0]
+    line = next((ln for ln in open("/proc/self/numa_maps")
+                 if ln.split()[0] == format(t.data_ptr(), "x")), "")
+    counts = {int(k): int(v) for k, v in re.findall(r"N(\d+)=(\d+)", line)}
+    if placed or counts:
+        assert all(s == node for s in placed), list(status)
+        assert set(counts) <= {node}, line
+    else:
+        # -ENOENT for every page and no per-node counts: not ordinary process memory
+        assert all(s == -2 for s in status), list(status)
+        assert "file=/dev/" in line, line
+
+
 def test_async_copy_round_trip_with_event_fencing():
     """H2D on one side stream, kernel on the compute stream, D2H on another."""
     from offload_adam_amd import _lib
