@@ -1,7 +1,7 @@
 /* liboffload_adam_copy_engines.so: an HSA tools library (loaded by the ROCr
  * runtime through HSA_TOOLS_LIB, before the first HIP call) that gives the
- * host->device and the device->host copies of the process one fixed SDMA
- * engine each.  It has no counterpart in the reference, whose copies go
+ * host->device and the device->host copies of the optimizer's pinned buffers
+ * (of the whole process until a range is registered) one fixed SDMA engine each.  It has no counterpart in the reference, whose copies go
  * through torch's non_blocking copies on two CUDA streams
  * (src/offload_adam/offload_adam.py:346-358 and :362-372) and rely on the CUDA
  * driver's copy engines; on MI355X the HIP runtime's per-copy engine choice has
@@ -19,6 +19,8 @@
  */
 #ifndef OFFLOAD_ADAM_COPY_ENGINES_H
 #define OFFLOAD_ADAM_COPY_ENGINES_H
+
+#include <stddef.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -43,6 +45,23 @@ void oa_copy_engines_stats(unsigned long long* h2d_copies, unsigned long long* d
  * engine (hsa_amd_memory_async_copy) and were sent to the fixed engines as well;
  * they are included in the per-direction counts above. */
 unsigned long long oa_copy_engines_unpinned_calls(void);
+
+/* Scope of the rewrite.  Until the first registration every pinned host<->device
+ * copy of the process is rewritten; from then on only copies whose host side
+ * lies inside a registered range [base, base + bytes) are, and all others keep
+ * the engine the HIP runtime chose.  The package's pinned allocator registers
+ * what it hands out and unregisters it on release.  Both return 0, or -1 for a
+ * null / empty range or a base that was never registered.  Thread-safe. */
+int oa_copy_engines_register_range(const void* base, size_t bytes);
+int oa_copy_engines_unregister_range(const void* base);
+
+/* 1 once a range has been registered in this process (the rewrite is limited
+ * to registered ranges), else 0. */
+int oa_copy_engines_scoped(void);
+
+/* Host<->device copies left to the runtime because their host side was outside
+ * every registered range. */
+unsigned long long oa_copy_engines_passed_by(void);
 
 #ifdef __cplusplus
 }

@@ -31,7 +31,9 @@ def _gpu_runtime_started():
 def install():
     """Put the tools library on ``HSA_TOOLS_LIB``.  Returns one of
     ``"installed"``, ``"off"`` (disabled by the environment), ``"missing"``
-    (library not built) or ``"late"`` (the GPU runtime is already up)."""
+    (library not built), ``"unusable_path"`` (the install path contains
+    whitespace, which ``HSA_TOOLS_LIB`` cannot express) or ``"late"`` (the GPU
+    runtime is already up)."""
     global _install_result
     if _install_result in ("installed", "off"):
         return _install_result
@@ -39,6 +41,9 @@ def install():
         _install_result = "off"
     elif not LIB_PATH.exists():
         _install_result = "missing"
+    elif any(ch.isspace() for ch in str(LIB_PATH)):
+        # HSA_TOOLS_LIB is a whitespace-separated list: such a path cannot be named in it
+        _install_result = "unusable_path"
     elif str(LIB_PATH) in os.environ.get("HSA_TOOLS_LIB", "").split():
         _install_result = "installed"
     elif _gpu_runtime_started():
@@ -50,15 +55,45 @@ def install():
     return _install_result
 
 
+_handle = None
+
+
+def _lib():
+    global _handle
+    if _handle is None and LIB_PATH.exists():
+        lib = ctypes.CDLL(str(LIB_PATH))  # same handle the runtime holds, if it loaded it
+        lib.oa_copy_engines_register_range.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+        lib.oa_copy_engines_register_range.restype = ctypes.c_int
+        lib.oa_copy_engines_unregister_range.argtypes = [ctypes.c_void_p]
+        lib.oa_copy_engines_unregister_range.restype = ctypes.c_int
+        _handle = lib
+    return _handle
+
+
+def register_range(ptr, nbytes):
+    """Tell the tools library that ``[ptr, ptr + nbytes)`` is an optimizer buffer:
+    from the first registration on, only copies to or from registered ranges are
+    put on the fixed engines.  No-op when the library is not built."""
+    lib = _lib()
+    if lib is not None:
+        lib.oa_copy_engines_register_range(ctypes.c_void_p(ptr), ctypes.c_size_t(nbytes))
+
+
+def unregister_range(ptr):
+    lib = _lib()
+    if lib is not None:
+        lib.oa_copy_engines_unregister_range(ctypes.c_void_p(ptr))
+
+
 def status():
     """What the tools library reports once the GPU runtime is up:
     ``{"install", "loaded", "active", "h2d_engine", "d2h_engine", "h2d_copies",
-    "d2h_copies", "rejected", "unpinned_calls"}``.  ``loaded`` is False when the runtime started
+    "d2h_copies", "rejected", "unpinned_calls", "scoped", "passed_by"}``.  ``loaded`` is False when the runtime started
     before :func:`install` ran (or the library is missing)."""
     out = {"install": _install_result, "loaded": False, "active": False}
     if not LIB_PATH.exists():
         return out
-    lib = ctypes.CDLL(str(LIB_PATH))  # same handle the runtime holds, if it loaded it
+    lib = _lib()
     lib.oa_copy_engines_loaded.restype = ctypes.c_int
     lib.oa_copy_engines_active.restype = ctypes.c_int
     lib.oa_copy_engines_config.restype = None
@@ -73,4 +108,8 @@ def status():
     out["h2d_copies"], out["d2h_copies"], out["rejected"] = a.value, b.value, c.value
     lib.oa_copy_engines_unpinned_calls.restype = ctypes.c_ulonglong
     out["unpinned_calls"] = lib.oa_copy_engines_unpinned_calls()
+    lib.oa_copy_engines_scoped.restype = ctypes.c_int
+    lib.oa_copy_engines_passed_by.restype = ctypes.c_ulonglong
+    out["scoped"] = bool(lib.oa_copy_engines_scoped())
+    out["passed_by"] = lib.oa_copy_engines_passed_by()
     return out

@@ -22,6 +22,14 @@
 // runtime rejects a rewritten call, the original call is made instead, and after
 // eight such rejections in a row the rewrite switches itself off.
 //
+// Scope.  Until a host range is registered (oa_copy_engines_register_range) every
+// pinned host<->device copy of the process is rewritten.  From the first
+// registration on, only copies whose host side lies inside a registered range
+// are: the optimizer's own buffers, which the package's pinned allocator
+// registers.  Copies of anybody else in the process (a data loader, torch's
+// pinned tensors) then keep the engine the HIP runtime chose and do not queue
+// behind 100 MB state transfers on the two fixed rings.
+//
 // Configuration (read once, at load):
 //   OFFLOAD_ADAM_COPY_ENGINES="<h2d mask>,<d2h mask>"   default "0x1,0x2"
 //   OFFLOAD_ADAM_COPY_ENGINES=off                       load, but rewrite nothing
@@ -34,9 +42,13 @@
 #include <hsa_ext_amd.h>
 #include <hsa_api_trace.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <shared_mutex>
+#include <vector>
 
 #include "offload_adam_copy_engines.h"
 
@@ -54,6 +66,35 @@ std::atomic<unsigned long long> n_h2d{0}, n_d2h{0}, n_rejected{0}, n_unpinned{0}
 std::atomic<int> rejected_in_a_row{0};
 constexpr int kMaxRejectedInARow = 8;
 
+// Registered host ranges, sorted by base; `scoped` is set by the first registration.
+struct Range {
+  uintptr_t base, end;
+};
+std::shared_mutex ranges_mutex;
+std::vector<Range> ranges;
+std::atomic<int> scoped{0};
+std::atomic<unsigned long long> n_passed_by{0};
+
+bool in_registered_range(const void* p) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  std::shared_lock<std::shared_mutex> lock(ranges_mutex);
+  auto it = std::upper_bound(ranges.begin(), ranges.end(), a,
+                             [](uintptr_t x, const Range& r) { return x < r.base; });
+  if (it == ranges.begin()) return false;
+  --it;
+  return a < it->end;
+}
+
+// Which fixed engine a copy goes to: 0 = leave it to the runtime.
+unsigned engine_for(const void* dst, bool dst_cpu, const void* src, bool src_cpu) {
+  if (src_cpu == dst_cpu) return 0;
+  if (scoped.load(std::memory_order_relaxed) && !in_registered_range(src_cpu ? src : dst)) {
+    n_passed_by.fetch_add(1, std::memory_order_relaxed);
+    return 0;
+  }
+  return src_cpu ? h2d_engine : d2h_engine;
+}
+
 bool single_bit(unsigned m) { return m != 0 && (m & (m - 1)) == 0 && m <= 0x8000u; }
 
 bool is_cpu(hsa_agent_t agent) {
@@ -68,9 +109,7 @@ hsa_status_t copy_on_fixed_engine(void* dst, hsa_agent_t dst_agent, const void* 
                                   hsa_amd_sdma_engine_id_t engine_id, bool force_copy_on_sdma) {
   if (active.load(std::memory_order_relaxed)) {
     const bool src_cpu = is_cpu(src_agent), dst_cpu = is_cpu(dst_agent);
-    unsigned want = 0;
-    if (src_cpu && !dst_cpu) want = h2d_engine;
-    else if (!src_cpu && dst_cpu) want = d2h_engine;
+    const unsigned want = engine_for(dst, dst_cpu, src, src_cpu);
     if (want != 0) {
       hsa_status_t st = real_copy_on_engine(dst, dst_agent, src, src_agent, size, num_dep_signals,
                                             dep_signals, completion_signal,
@@ -100,9 +139,7 @@ hsa_status_t copy_without_engine(void* dst, hsa_agent_t dst_agent, const void* s
                                  hsa_signal_t completion_signal) {
   if (active.load(std::memory_order_relaxed)) {
     const bool src_cpu = is_cpu(src_agent), dst_cpu = is_cpu(dst_agent);
-    unsigned want = 0;
-    if (src_cpu && !dst_cpu) want = h2d_engine;
-    else if (!src_cpu && dst_cpu) want = d2h_engine;
+    const unsigned want = engine_for(dst, dst_cpu, src, src_cpu);
     if (want != 0) {
       n_unpinned.fetch_add(1, std::memory_order_relaxed);
       hsa_status_t st = real_copy_on_engine(dst, dst_agent, src, src_agent, size, num_dep_signals,
@@ -166,6 +203,34 @@ extern "C" void oa_copy_engines_config(unsigned* h2d_mask, unsigned* d2h_mask) {
 }
 
 extern "C" unsigned long long oa_copy_engines_unpinned_calls(void) { return n_unpinned.load(); }
+
+extern "C" int oa_copy_engines_register_range(const void* base, size_t bytes) {
+  if (!base || bytes == 0) return -1;
+  const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+  std::unique_lock<std::shared_mutex> lock(ranges_mutex);
+  auto it = std::lower_bound(ranges.begin(), ranges.end(), b,
+                             [](const Range& r, uintptr_t x) { return r.base < x; });
+  if (it != ranges.end() && it->base == b) it->end = b + bytes;
+  else ranges.insert(it, Range{b, b + bytes});
+  scoped.store(1, std::memory_order_relaxed);
+  return 0;
+}
+
+extern "C" int oa_copy_engines_unregister_range(const void* base) {
+  const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+  std::unique_lock<std::shared_mutex> lock(ranges_mutex);
+  for (auto it = ranges.begin(); it != ranges.end(); ++it) {
+    if (it->base == b) {
+      ranges.erase(it);
+      return 0;
+    }
+  }
+  return -1;
+}
+
+extern "C" int oa_copy_engines_scoped(void) { return scoped.load(); }
+
+extern "C" unsigned long long oa_copy_engines_passed_by(void) { return n_passed_by.load(); }
 
 extern "C" void oa_copy_engines_stats(unsigned long long* h2d_copies, unsigned long long* d2h_copies,
                                       unsigned long long* rejected) {

@@ -466,7 +466,12 @@ class OffloadAdam(Optimizer):
                 self._offload_params[0].device
             )
             if self.verbose > 0:
+                from . import _runtime_env
+
                 print(f"Transfer streams: {self.transfer_stream_report}")
+                print(f"Process environment set at import: {_runtime_env.prepare()} "
+                      "(HSA_TOOLS_LIB gets the copy-engine library, GPU_MAX_HW_QUEUES the "
+                      "number of hardware queues)")
         else:
             self.h2d_stream = torch.cuda.Stream()
             self.d2h_stream = torch.cuda.Stream()
@@ -631,6 +636,8 @@ class OffloadAdam(Optimizer):
             "late": "offload_adam_amd was imported after the GPU runtime had started",
             "missing": f"{_copy_engines.LIB_PATH.name} is not built "
                        "(python -m offload_adam_amd._build)",
+            "unusable_path": f"the path of {_copy_engines.LIB_PATH.name} contains whitespace, "
+                             "which HSA_TOOLS_LIB cannot name",
         }.get(st["install"], "the ROCr runtime did not load it from HSA_TOOLS_LIB")
         warnings.warn(
             "OffloadAdam: host<->device copies are not pinned to fixed SDMA engines ("

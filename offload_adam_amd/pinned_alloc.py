@@ -22,7 +22,7 @@ from pathlib import Path
 
 import torch
 
-from . import _lib
+from . import _copy_engines, _lib
 
 _PAGE_SIZE = 4096
 _MPOL_SYSCALL_PROBED = None
@@ -106,9 +106,12 @@ def _alloc(size, numa_target):
             f"{_lib.error_string(code)}"
         )
     ptr = out.value
+    # copies to and from this block go to the fixed SDMA engines; anybody else's do not
+    _copy_engines.register_range(ptr, size)
 
     def cleanup():
         try:
+            _copy_engines.unregister_range(ptr)
             lib.oa_pinned_free(ctypes.c_void_p(ptr))
         except Exception:
             pass

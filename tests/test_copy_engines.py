@@ -26,7 +26,9 @@ def test_library_exports_header_symbols_and_tool_entry_points():
     lib = ctypes.CDLL(str(_copy_engines.LIB_PATH))
     names = declared()
     assert names == ["oa_copy_engines_active", "oa_copy_engines_config", "oa_copy_engines_loaded",
-                     "oa_copy_engines_stats", "oa_copy_engines_unpinned_calls"]
+                     "oa_copy_engines_passed_by", "oa_copy_engines_register_range",
+                     "oa_copy_engines_scoped", "oa_copy_engines_stats",
+                     "oa_copy_engines_unpinned_calls", "oa_copy_engines_unregister_range"]
     for name in names + ["OnLoad", "OnUnload"]:
         assert hasattr(lib, name), name
 
@@ -40,6 +42,38 @@ def test_status_without_runtime_reports_not_loaded():
     assert st["active"] is False
     assert (st["h2d_engine"], st["d2h_engine"]) == (1, 2)
     assert st["h2d_copies"] == st["d2h_copies"] == st["rejected"] == 0
+
+
+def test_range_registry_in_a_process_of_its_own():
+    """Registering switches the library to its scoped mode; bases are unique keys."""
+    code = (
+        "import ctypes; from offload_adam_amd import _copy_engines as c\n"
+        "lib = c._lib(); lib.oa_copy_engines_scoped.restype = ctypes.c_int\n"
+        "a = lib.oa_copy_engines_scoped()\n"
+        "r = [lib.oa_copy_engines_register_range(ctypes.c_void_p(0x10000), 4096),\n"
+        "     lib.oa_copy_engines_register_range(ctypes.c_void_p(0x10000), 8192),\n"
+        "     lib.oa_copy_engines_register_range(ctypes.c_void_p(0x40000), 4096),\n"
+        "     lib.oa_copy_engines_register_range(None, 4096),\n"
+        "     lib.oa_copy_engines_register_range(ctypes.c_void_p(0x50000), 0)]\n"
+        "u = [lib.oa_copy_engines_unregister_range(ctypes.c_void_p(0x10000)),\n"
+        "     lib.oa_copy_engines_unregister_range(ctypes.c_void_p(0x10000)),\n"
+        "     lib.oa_copy_engines_unregister_range(ctypes.c_void_p(0x40000))]\n"
+        "print(a, r, u, lib.oa_copy_engines_scoped())")
+    assert _run(code) == "0 [0, 0, 0, -1, -1] [0, -1, 0] 1"
+
+
+def test_a_path_with_whitespace_is_reported_not_installed(monkeypatch, tmp_path):
+    from offload_adam_amd import _copy_engines
+
+    spaced = tmp_path / "with space" / "liboffload_adam_copy_engines.so"
+    spaced.parent.mkdir()
+    spaced.write_bytes(b"")
+    monkeypatch.setattr(_copy_engines, "LIB_PATH", spaced)
+    monkeypatch.setattr(_copy_engines, "_install_result", None)
+    monkeypatch.delenv("OFFLOAD_ADAM_COPY_ENGINES", raising=False)
+    before = os.environ.get("HSA_TOOLS_LIB")
+    assert _copy_engines.install() == "unusable_path"
+    assert os.environ.get("HSA_TOOLS_LIB") == before
 
 
 def _run(code, **env):
@@ -103,6 +137,19 @@ def test_copies_run_on_the_fixed_engines_and_move_the_right_bytes():
     assert st1["h2d_copies"] - st0["h2d_copies"] >= 4
     assert st1["d2h_copies"] - st0["d2h_copies"] >= 4
     assert st1["rejected"] == 0 and st1["active"]
+    # the package's pinned buffers are registered, so the rewrite is scoped to them:
+    # copies of torch's own pinned tensors keep the engine the runtime picks
+    assert st1["scoped"]
+    other = torch.empty(n, dtype=torch.int32).pin_memory()
+    other.copy_(host_in)
+    for _ in range(3):
+        dev = other.to("cuda", non_blocking=True)
+        back = dev.to("cpu", non_blocking=True)
+        torch.cuda.synchronize()
+        assert torch.equal(back, host_in)
+    st2 = _copy_engines.status()
+    assert st2["passed_by"] - st1["passed_by"] >= 3
+    assert st2["h2d_copies"] == st1["h2d_copies"]
 
 
 def test_roctx_ranges_are_off_by_default_and_load_on_request():
