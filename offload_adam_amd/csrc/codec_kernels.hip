@@ -15,6 +15,8 @@
 // Each codec has a fast path (cols % 8 == 0, 16-byte aligned rows, power-of-two
 // group) and a generic path (one lane per group, any shape and alignment).
 
+#include <type_traits>
+
 #include "oa_common.hpp"
 
 #pragma clang fp contract(off)
@@ -262,6 +264,126 @@ __device__ __forceinline__ int64_t octet_elem(int64_t o, int64_t opr, int64_t st
   return row * stride + (o - row * opr) * 8;
 }
 
+// ---------------------------------------------------------------- quads
+// Encoders of row-contiguous matrices give a lane a "quad": 32 consecutive
+// elements (four octets).  Global loads stay coalesced - in trip k a wave reads
+// octets 64k .. 64k+63 of its 256-octet chunk, 1 KiB per instruction - and the
+// octets change hands through LDS: written where they were loaded, read back four
+// in a row.  (Loading a lane's 64 contiguous bytes directly, 64 bytes apart from
+// its neighbour's, measured 2.3x slower on the NF4 encoder.)  Slot
+// (o & ~15) | ((o + (o >> 4)) & 15) of octet o keeps both the 16-byte writes and
+// the 16-byte reads of eight consecutive lanes on distinct bank groups.
+constexpr int kQuadT = 256;
+__device__ __forceinline__ int quad_slot(int o) { return (o & ~15) | ((o + (o >> 4)) & 15); }
+
+template <int DT>
+__device__ __forceinline__ void unpack16(const u32x4 w, float (&x)[8]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (DT == OA_BF16) {
+      x[2 * k] = bf16lo_to_f32(w[k]);
+      x[2 * k + 1] = bf16hi_to_f32(w[k]);
+    } else {
+      x[2 * k] = f16_bits_to_f32(w[k] & 0xFFFFu);
+      x[2 * k + 1] = f16_bits_to_f32(w[k] >> 16);
+    }
+  }
+}
+
+// LDS a workgroup of kQuadT lanes needs: one 16-byte plane per octet for 16-bit
+// sources, two for fp32.
+template <int SRC>
+constexpr int quad_lds_slots() { return (SRC == OA_F32 ? 2 : 1) * kQuadT * 4; }
+
+// Leaves the lane's quad (first element 32 * (q0 + threadIdx.x) of the flat
+// matrix) in x.  `octets` = octets of the whole matrix; quads beyond it read as
+// zero.  Contains a workgroup barrier: every lane of the workgroup calls it.
+template <int SRC>
+__device__ __forceinline__ void quad_fetch(const void* __restrict__ src, int64_t q0,
+                                           int64_t octets, u32x4* lds, float (&x)[4][8]) {
+  constexpr int P = SRC == OA_F32 ? 2 : 1;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  u32x4* mine = lds + wave * (P * 256);
+  const int64_t o0 = (q0 + wave * kWave) * 4;  // first octet of this wave's chunk
+  u32x4 raw[4][P];
+  const char* base = static_cast<const char*>(src) + (o0 + lane) * (16 * P);
+  if ((q0 + kQuadT) * 4 <= octets) {
+    // every lane of the workgroup is in range (a scalar branch): the loads carry no
+    // guards, so all of them are in flight before the first is waited for
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int pl = 0; pl < P; ++pl)
+        raw[k][pl] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4*>(base + (int64_t)k * (64 * 16 * P)) + pl);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool in = o0 + 64 * k + lane < octets;
+      // the last workgroup: out-of-range lanes re-read the matrix's first octet
+      const u32x4* p = reinterpret_cast<const u32x4*>(
+          in ? base + (int64_t)k * (64 * 16 * P) : static_cast<const char*>(src));
+#pragma unroll
+      for (int pl = 0; pl < P; ++pl) {
+        const u32x4 v = __builtin_nontemporal_load(p + pl);
+        raw[k][pl] = in ? v : u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int pl = 0; pl < P; ++pl) mine[pl * 256 + quad_slot(64 * k + lane)] = raw[k][pl];
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int slot = quad_slot(4 * lane + j);
+    if (SRC == OA_F32) {
+      const u32x4 a = mine[slot], b = mine[256 + slot];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x[j][i] = __uint_as_float(a[i]);
+        x[j][4 + i] = __uint_as_float(b[i]);
+      }
+    } else {
+      unpack16<SRC>(mine[slot], x[j]);
+    }
+  }
+}
+
+// N trips of a row: lane t takes octets t, t + kT, ..., all loads issued before
+// the first value is converted; trips N .. kRowCache-1 read as zero.
+template <int SRC, int N, int R>
+__device__ __forceinline__ void load_trips(const void* lane_base, float (&x)[R][8]) {
+  constexpr int P = SRC == OA_F32 ? 2 : 1;
+  u32x4 raw[N][P];
+#pragma unroll
+  for (int k = 0; k < N; ++k)
+#pragma unroll
+    for (int pl = 0; pl < P; ++pl)
+      raw[k][pl] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4*>(static_cast<const char*>(lane_base) +
+                                         (int64_t)k * kT * 16 * P) + pl);
+#pragma unroll
+  for (int k = 0; k < R; ++k) {
+    if (k < N) {
+      if constexpr (SRC == OA_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          x[k][i] = __uint_as_float(raw[k < N ? k : 0][0][i]);
+          x[k][4 + i] = __uint_as_float(raw[k < N ? k : 0][P - 1][i]);
+        }
+      } else {
+        unpack16<SRC>(raw[k < N ? k : 0][0], x[k]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[k][i] = 0.0f;
+    }
+  }
+}
+
 // ------------------------------------------------------------------- int8
 
 __device__ __forceinline__ int32_t q_int8(float x, float inv) {
@@ -293,24 +415,49 @@ quant_int8_kernel(const void* __restrict__ src, int64_t stride, int64_t cols,
   float xc[kRowCache][8];
   float a = 0.0f;
   if (cached) {
-    // loads of kI8Batch octets at a time before their stores (fused source)
-#pragma unroll
-    for (int kb = 0; kb < kRowCache; kb += kI8Batch) {
-      AdamRaw raw[kI8Batch];
-#pragma unroll
-      for (int k = kb; k < kb + kI8Batch; ++k) {
-        const int64_t o = threadIdx.x + (int64_t)k * kT;
-        if (o < octets) {
-          fetch8_begin<SRC>(src, ad, base + o * 8, raw[k - kb], xc[k]);
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) xc[k][j] = 0.0f;
+    bool loaded = false;
+    if constexpr (SRC != kSrcAdam) {
+      // A row of whole trips (octets % kT == 0): one straight-line run of
+      // unguarded loads per trip count, all in flight before the first convert.
+      // (A guarded load - or one inside any branch that also converts it - is
+      // waited for before the next is issued: one load in flight per wave.)
+      if (octets % kT == 0) {
+        loaded = true;
+        const void* at = static_cast<const char*>(src) +
+                         (base + (int64_t)threadIdx.x * 8) * (SRC == OA_F32 ? 4 : 2);
+        switch ((int)(octets / kT)) {
+          case 1: load_trips<SRC, 1>(at, xc); break;
+          case 2: load_trips<SRC, 2>(at, xc); break;
+          case 3: load_trips<SRC, 3>(at, xc); break;
+          case 4: load_trips<SRC, 4>(at, xc); break;
+          case 5: load_trips<SRC, 5>(at, xc); break;
+          case 6: load_trips<SRC, 6>(at, xc); break;
+          case 7: load_trips<SRC, 7>(at, xc); break;
+          case 8: load_trips<SRC, 8>(at, xc); break;
+          default: loaded = false; break;
         }
       }
+    }
+    if (!loaded) {
+      // loads of kI8Batch octets at a time before their stores (fused source)
 #pragma unroll
-      for (int k = kb; k < kb + kI8Batch; ++k) {
-        const int64_t o = threadIdx.x + (int64_t)k * kT;
-        if (o < octets) fetch8_end<SRC>(ad, base + o * 8, raw[k - kb], xc[k]);
+      for (int kb = 0; kb < kRowCache; kb += kI8Batch) {
+        AdamRaw raw[kI8Batch];
+#pragma unroll
+        for (int k = kb; k < kb + kI8Batch; ++k) {
+          const int64_t o = threadIdx.x + (int64_t)k * kT;
+          if (o < octets) {
+            fetch8_begin<SRC>(src, ad, base + o * 8, raw[k - kb], xc[k]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xc[k][j] = 0.0f;
+          }
+        }
+#pragma unroll
+        for (int k = kb; k < kb + kI8Batch; ++k) {
+          const int64_t o = threadIdx.x + (int64_t)k * kT;
+          if (o < octets) fetch8_end<SRC>(ad, base + o * 8, raw[k - kb], xc[k]);
+        }
       }
     }
 #pragma unroll
@@ -413,6 +560,8 @@ __device__ __forceinline__ uint32_t q_int4_word(const float (&x)[8], float inv) 
 }
 
 constexpr int kI4RowsQ = 64;   // rows of one LDS tile, encoder
+constexpr int kI4PitchQ = 68;  // words per LDS row of it: 16-byte aligned rows, and the
+                               // writes of a wave (16 word columns x 4 rows) hit 64 banks
 constexpr int kI4RowsD = 128;  // rows of one LDS tile, decoder
 constexpr int kI4Chunk = 4;    // decoder: packed words a lane fetches per trip
 // Consecutive workgroups walk along the row (group index fastest): the tiles in
@@ -444,8 +593,8 @@ quant_int4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, in
                   const AdamSrc ad) {
   extern __shared__ uint32_t i4_lds[];
   const int wpr = WPR ? WPR : (group >> 3);
-  uint32_t* words = i4_lds;                                  // [wpr][kI4RowsQ + 1]
-  float* scale_s = reinterpret_cast<float*>(words + wpr * (kI4RowsQ + 1));
+  uint32_t* words = i4_lds;                                  // [wpr][kI4PitchQ]
+  float* scale_s = reinterpret_cast<float*>(words + wpr * kI4PitchQ);
 #if OA_I4_GROUP_FASTEST
   const int64_t r0 = (int64_t)blockIdx.y * kI4RowsQ;
   const int64_t gi = blockIdx.x;
@@ -456,25 +605,66 @@ quant_int4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, in
   const int rows_per_pass = kT / wpr;
   const int k = threadIdx.x % wpr;
   const int rsub = threadIdx.x / wpr;
-  for (int pr = 0; pr < kI4RowsQ; pr += rows_per_pass) {
-    const int rl = pr + rsub;
-    const int64_t row = r0 + rl;
-    float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (rl < kI4RowsQ && row < rows)
-      fetch8<SRC>(src, ad, row * stride + gi * group + k * 8, x);
+  // A tile that lies wholly inside the matrix (a scalar condition) loads without
+  // per-lane guards; a guarded load sits in a divergent branch and is waited for
+  // before the next one is issued.
+  const bool full = r0 + kI4RowsQ <= rows;
+  auto encode_row = [&](const float (&x)[8], int rl) {
     const float absmax = group_max(absmax8(x), wpr);
     const float scale = absmax / 8.0f;
     const float inv = 1.0f / fmaxf(scale, kEps);
     if (rl < kI4RowsQ) {
-      words[k * (kI4RowsQ + 1) + rl] = q_int4_word(x, inv);
+      words[k * kI4PitchQ + rl] = q_int4_word(x, inv);
       if (k == 0) scale_s[rl] = scale;
+    }
+  };
+  if constexpr (WPR != 0 && SRC != kSrcAdam) {
+    // plain sources: the loads of every row pass are issued before the first is used
+    constexpr int kPasses = kI4RowsQ / (kT / WPR);
+    float x[kPasses][8];
+    if (full) {
+#pragma unroll
+      for (int p = 0; p < kPasses; ++p)
+        load8<SRC>(src, (r0 + p * (kT / WPR) + rsub) * stride + gi * group + k * 8, x[p]);
+    } else {
+#pragma unroll
+      for (int p = 0; p < kPasses; ++p) {
+        const int64_t row = r0 + p * (kT / WPR) + rsub;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[p][i] = 0.0f;
+        if (row < rows) load8<SRC>(src, row * stride + gi * group + k * 8, x[p]);
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) encode_row(x[p], p * (kT / WPR) + rsub);
+  } else {
+    for (int pr = 0; pr < kI4RowsQ; pr += rows_per_pass) {
+      const int rl = pr + rsub;
+      const int64_t row = r0 + rl;
+      float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (full && rl < kI4RowsQ) {
+        fetch8<SRC>(src, ad, row * stride + gi * group + k * 8, x);
+      } else if (rl < kI4RowsQ && row < rows) {
+        fetch8<SRC>(src, ad, row * stride + gi * group + k * 8, x);
+      }
+      encode_row(x, rl);
     }
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < wpr * kI4RowsQ; idx += kT) {
-    const int kk = idx / kI4RowsQ, rl = idx % kI4RowsQ;
-    if (r0 + rl < rows)
-      qweight[(gi * wpr + kk) * rows + r0 + rl] = (int32_t)words[kk * (kI4RowsQ + 1) + rl];
+  if (full && (rows & 3) == 0) {
+    // 16 bytes of the transposed payload per lane: four consecutive rows of one word column
+    for (int idx = threadIdx.x; idx < wpr * (kI4RowsQ / 4); idx += kT) {
+      const int kk = idx / (kI4RowsQ / 4), r4 = idx % (kI4RowsQ / 4);
+      const u32x4 w = *reinterpret_cast<const u32x4*>(words + kk * kI4PitchQ + 4 * r4);
+      __builtin_nontemporal_store(
+          w, reinterpret_cast<u32x4*>(qweight + (gi * wpr + kk) * rows + r0 + 4 * r4));
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < wpr * kI4RowsQ; idx += kT) {
+      const int kk = idx / kI4RowsQ, rl = idx % kI4RowsQ;
+      if (r0 + rl < rows)
+        qweight[(gi * wpr + kk) * rows + r0 + rl] = (int32_t)words[kk * kI4PitchQ + rl];
+    }
   }
   if (threadIdx.x < kI4RowsQ && r0 + threadIdx.x < rows)
     store_scale(scales, sdt, gi * rows + r0 + threadIdx.x, scale_s[threadIdx.x]);
@@ -679,6 +869,96 @@ __device__ __forceinline__ uint32_t nf4_pack8(const float (&x)[8], float inv16, 
   return w;
 }
 
+// The same count with one fp32 add in place of add, convert and two clamps: the
+// low mantissa bits of m + (2^23 + 16) are round-half-even(m + 16), an integer in
+// [0, 32] for every finite input (|m| <= 16 (1 + 2^-23)).  Buckets are again
+// monotone in n and one unit of m wide, so each holds at most one threshold; 64
+// entries, because a NaN leaves arbitrary low bits (entries above 32 give code 0,
+// as bucket 0 does for the canonical NaN: the reference's argmin over NaN
+// distances is 0 as well).
+constexpr float kNf4Magic = 8388624.0f;  // 2^23 + 16
+constexpr int nf4_rbucket(float m) {
+  return (int)(__builtin_bit_cast(uint32_t, m + kNf4Magic) & 63u);
+}
+struct Nf4RBuckets {
+  uint32_t own16[64];
+  uint32_t below[64];
+};
+constexpr Nf4RBuckets make_nf4_rbuckets() {
+  Nf4RBuckets t{};
+  for (int k = 0; k < 64; ++k) {
+    t.own16[k] = 0x7F800000u;
+    t.below[k] = 0;
+  }
+  for (int i = 0; i < 15; ++i) {
+    const float t16 = __builtin_bit_cast(float, kNf4T[i]) * 16.0f;
+    const int b = nf4_rbucket(t16);
+    t.own16[b] = __builtin_bit_cast(uint32_t, t16);
+    for (int k = b + 1; k <= 32; ++k) t.below[k] += 1;
+  }
+  return t;
+}
+constexpr bool nf4_rbuckets_distinct() {
+  int last = -1;
+  for (int i = 0; i < 15; ++i) {
+    const int b = nf4_rbucket(__builtin_bit_cast(float, kNf4T[i]) * 16.0f);
+    if (b <= last || b > 32) return false;
+    last = b;
+  }
+  return nf4_rbucket(-16.000002f) == 0 && nf4_rbucket(16.000002f) == 32;
+}
+static_assert(nf4_rbuckets_distinct(), "two NF4 thresholds share a rounded bucket");
+__device__ const Nf4RBuckets kNf4RBuckets = make_nf4_rbuckets();
+
+__device__ __forceinline__ uint32_t nf4_code16r(float m, const u32x2* lut) {
+  const u32x2 e = lut[__float_as_uint(m + kNf4Magic) & 63u];
+  return e[1] + (uint32_t)(m >= __uint_as_float(e[0]));
+}
+
+__device__ __forceinline__ uint32_t nf4_pack8r(const float (&x)[8], float inv16, const u32x2* lut) {
+  uint32_t w = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t hi = nf4_code16r(x[2 * j] * inv16, lut);
+    const uint32_t lo = nf4_code16r(x[2 * j + 1] * inv16, lut);
+    w |= ((hi << 4) | lo) << (8 * j);
+  }
+  return w;
+}
+
+// Row-contiguous matrices whose blocks are whole "quads": a lane owns 32
+// consecutive elements (four octets), LPB lanes share a block (block = 32 LPB).
+// Against one octet per lane and trip: the block maximum needs log2(LPB) shuffle
+// steps per 32 elements instead of three per octet, the correctly rounded
+// reciprocal is taken once per 32 elements, and the codes leave as one 16-byte
+// store per lane (1 KiB per wave instruction; the maxima as one run of floats).
+// The quad arrives through quad_fetch().
+template <int SRC, int LPB>
+__global__ void __launch_bounds__(kQuadT)
+quant_nf4_quad_kernel(const void* __restrict__ src, int64_t quads, int lpb_arg, int lpb_shift_arg,
+                      u32x4* __restrict__ packed, float* __restrict__ absmax_out) {
+  const int lpb = LPB ? LPB : lpb_arg;
+  const int lpb_shift = LPB ? __builtin_ctz((unsigned)(LPB ? LPB : 1)) : lpb_shift_arg;
+  __shared__ u32x2 lut[64];
+  __shared__ u32x4 stage[quad_lds_slots<SRC>()];
+  if (threadIdx.x < 64)
+    lut[threadIdx.x] = u32x2{kNf4RBuckets.own16[threadIdx.x], kNf4RBuckets.below[threadIdx.x]};
+  const int64_t q0 = (int64_t)blockIdx.x * kQuadT;
+  const int64_t q = q0 + threadIdx.x;
+  float x[4][8];
+  quad_fetch<SRC>(src, q0, quads * 4, stage, x);  // its barrier also covers the table
+  float a = fmaxf(fmaxf(absmax8(x[0]), absmax8(x[1])), fmaxf(absmax8(x[2]), absmax8(x[3])));
+  a = group_max(a, lpb);
+  const float inv16 = (1.0f / fmaxf(a, kEps)) * 16.0f;
+  u32x4 w;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) w[j] = nf4_pack8r(x[j], inv16, lut);
+  if (q < quads) {
+    __builtin_nontemporal_store(w, packed + q);
+    if ((threadIdx.x & (lpb - 1)) == 0) absmax_out[q >> lpb_shift] = a;
+  }
+}
+
 // Flat over octets; lpg = block/8 lanes share a block (power of two <= 64).
 // LPG != 0: that many lanes per block, known at compile time (8 = the usual
 // 64-element block): the shuffle ladder of the block maximum unrolls.
@@ -857,9 +1137,20 @@ nvfp4_amax_partial_kernel(const void* __restrict__ src, int64_t stride, int64_t 
     const int64_t opr = cols >> 3, total = rows * opr;
     const bool flat = stride == cols;
     const int64_t tile = SRC == kSrcAdam ? xcd_tile<kCodecXcdChunk>(blockIdx.x) : blockIdx.x;
-    int64_t o = tile * kT * kAmaxUnroll + threadIdx.x;
-    for (; o < total; o += step * kAmaxUnroll) {
+    int64_t ob = tile * kT * kAmaxUnroll;  // the trip's first octet (the same in every lane)
+    for (; ob < total; ob += step * kAmaxUnroll) {
+      const int64_t o = ob + threadIdx.x;
       float x[kAmaxUnroll][8];
+      // every lane of every trip in range (a scalar condition): loads without guards,
+      // all in flight together
+      if (flat && SRC != kSrcAdam && ob + (int64_t)kAmaxUnroll * kT <= total) {
+#pragma unroll
+        for (int k = 0; k < kAmaxUnroll; ++k)
+          fetch8<SRC>(src, ad, (o + (int64_t)k * kT) * 8, x[k]);
+#pragma unroll
+        for (int k = 0; k < kAmaxUnroll; ++k) a = fmaxf(a, absmax8(x[k]));
+        continue;
+      }
 #pragma unroll
       for (int k = 0; k < kAmaxUnroll; ++k) {
         const int64_t ok = o + (int64_t)k * kT;
@@ -980,6 +1271,39 @@ quant_nvfp4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, i
     } else if ((lane & 1) == 0) {
       scale8[o >> 1] = (uint8_t)s8;
     }
+  }
+}
+
+// Row-contiguous matrices, 32 consecutive elements (two 16-element blocks) per
+// lane: block maxima need no shuffle, each block's scale arithmetic runs once
+// (not once in each of the two lanes that share a block in the octet kernel), and
+// the codes leave as one 16-byte store, the two scale bytes as one 2-byte store.
+template <int SRC>
+__global__ void __launch_bounds__(kQuadT)
+quant_nvfp4_quad_kernel(const void* __restrict__ src, int64_t quads, u32x4* __restrict__ packed,
+                        uint16_t* __restrict__ scale16, const float* __restrict__ gs_ptr) {
+  __shared__ u32x4 stage[quad_lds_slots<SRC>()];
+  const int64_t q0 = (int64_t)blockIdx.x * kQuadT;
+  const int64_t q = q0 + threadIdx.x;
+  float x[4][8];
+  quad_fetch<SRC>(src, q0, quads * 4, stage, x);
+  const float gs = *gs_ptr;
+  const float inv_global = 1.0f / gs;
+  u32x4 w;
+  uint32_t s2 = 0;
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const float amax = fmaxf(absmax8(x[2 * b]), absmax8(x[2 * b + 1]));
+    const uint32_t s8 = nvfp4_block_scale(amax, inv_global);
+    const float eff = e4m3fn_bits_to_f32(s8) * gs;
+    const float inv_eff = 1.0f / fmaxf(eff, kEps);
+    w[2 * b] = nvfp4_pack8(x[2 * b], inv_eff);
+    w[2 * b + 1] = nvfp4_pack8(x[2 * b + 1], inv_eff);
+    s2 |= s8 << (8 * b);
+  }
+  if (q < quads) {
+    __builtin_nontemporal_store(w, packed + q);
+    scale16[q] = (uint16_t)s2;
   }
 }
 
@@ -1162,7 +1486,7 @@ extern "C" int oa_quant_int4(const void* src, int src_dtype, int64_t src_row_str
                     group <= 512 && i4_grid_ok((rows + kI4RowsQ - 1) / kI4RowsQ, ng);
   if (fast) {
     const int wpr = (int)(group / 8);
-    const size_t lds = (size_t)wpr * (kI4RowsQ + 1) * 4 + kI4RowsQ * 4;
+    const size_t lds = (size_t)wpr * kI4PitchQ * 4 + kI4RowsQ * 4;
     const dim3 grid = i4_grid((unsigned)((rows + kI4RowsQ - 1) / kI4RowsQ), (unsigned)ng);
     OA_DISPATCH_DT(src_dtype, OA_DISPATCH_WPR(
         wpr, hipLaunchKernelGGL((quant_int4_kernel<DT, W>), grid, dim3(kT), lds, s, src,
@@ -1223,7 +1547,19 @@ extern "C" int oa_quant_nf4(const void* src, int src_dtype, int64_t src_row_stri
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool fast = rows_vec(src, src_dtype, src_row_stride, cols) && block % 8 == 0 &&
                     pow2(block / 8) && block <= 512 && aligned_to(packed, 4);
-  if (fast) {
+  // whole 32-element quads in one contiguous run, 16-byte aligned stores
+  const bool quad = fast && (src_row_stride == cols || rows <= 1) && block % 32 == 0 &&
+                    pow2(block / 32) && block <= 2048 && aligned_to(packed, 16);
+  if (quad) {
+    const int64_t quads = rows * cols / 32;
+    const int lpb = (int)(block / 32);
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL((block == 64 ? quant_nf4_quad_kernel<DT, 2>
+                                                   : quant_nf4_quad_kernel<DT, 0>),
+                                      dim3((unsigned)((quads + kQuadT - 1) / kQuadT)),
+                                      dim3(kQuadT), 0, s, src, quads, lpb, log2i(lpb),
+                                      static_cast<u32x4*>(packed), static_cast<float*>(absmax)));
+  } else if (fast) {
     OA_DISPATCH_DT(src_dtype,
                    hipLaunchKernelGGL((block == 64 ? quant_nf4_kernel<DT, 8> : quant_nf4_kernel<DT, 0>), dim3(blocks_oct(rows * (cols / 8))),
                                       dim3(kT), 0, s, src, src_row_stride, rows, cols,
@@ -1297,7 +1633,16 @@ extern "C" int oa_quant_nvfp4(const void* src, int src_dtype, int64_t src_row_st
                      static_cast<float*>(global_scale));
   rc = launch_status();
   if (rc || rows * cols == 0) return rc;
-  if (vec && aligned_to(packed, 4) && aligned_to(block_scale, 4)) {
+  if (vec && (src_row_stride == cols || rows <= 1) && (rows * cols) % 32 == 0 &&
+      aligned_to(packed, 16) && aligned_to(block_scale, 2)) {
+    const int64_t quads = rows * cols / 32;
+    OA_DISPATCH_DT(src_dtype,
+                   hipLaunchKernelGGL(quant_nvfp4_quad_kernel<DT>,
+                                      dim3((unsigned)((quads + kQuadT - 1) / kQuadT)),
+                                      dim3(kQuadT), 0, s, src, quads, static_cast<u32x4*>(packed),
+                                      static_cast<uint16_t*>(block_scale),
+                                      static_cast<const float*>(global_scale)));
+  } else if (vec && aligned_to(packed, 4) && aligned_to(block_scale, 4)) {
     OA_DISPATCH_DT(src_dtype,
                    hipLaunchKernelGGL(quant_nvfp4_kernel<DT>, dim3(blocks_oct(rows * (cols / 8))),
                                       dim3(kT), 0, s, src, src_row_stride, rows, cols,
@@ -1428,7 +1773,7 @@ extern "C" int oa_adam_requant_int4(const void* grad, void* exp_avg, void* exp_a
   if (!aligned_to(qweight, 4) || !aligned_to(scales, (uintptr_t)esize(scale_dtype)))
     return OA_EALIGN;
   const int wpr = (int)(group / 8);
-  const size_t lds = (size_t)wpr * (kI4RowsQ + 1) * 4 + kI4RowsQ * 4;
+  const size_t lds = (size_t)wpr * kI4PitchQ * 4 + kI4RowsQ * 4;
   const dim3 grid = i4_grid((unsigned)((rows + kI4RowsQ - 1) / kI4RowsQ), (unsigned)(cols / group));
   OA_DISPATCH_WPR(wpr, hipLaunchKernelGGL((quant_int4_kernel<kSrcAdam, W>), grid, dim3(kT), lds,
                                           static_cast<hipStream_t>(stream), nullptr, cols, rows,
