@@ -273,7 +273,10 @@ __device__ __forceinline__ int64_t octet_elem(int64_t o, int64_t opr, int64_t st
 // its neighbour's, measured 2.3x slower on the NF4 encoder.)  Slot
 // (o & ~15) | ((o + (o >> 4)) & 15) of octet o keeps both the 16-byte writes and
 // the 16-byte reads of eight consecutive lanes on distinct bank groups.
-constexpr int kQuadT = 256;
+#ifndef OA_QUAD_T
+#define OA_QUAD_T 64
+#endif
+constexpr int kQuadT = OA_QUAD_T;  // lanes of a quad-encoder workgroup
 __device__ __forceinline__ int quad_slot(int o) { return (o & ~15) | ((o + (o >> 4)) & 15); }
 
 template <int DT>
@@ -295,18 +298,31 @@ __device__ __forceinline__ void unpack16(const u32x4 w, float (&x)[8]) {
 template <int SRC>
 constexpr int quad_lds_slots() { return (SRC == OA_F32 ? 2 : 1) * kQuadT * 4; }
 
-// Leaves the lane's quad (first element 32 * (q0 + threadIdx.x) of the flat
-// matrix) in x.  `octets` = octets of the whole matrix; quads beyond it read as
-// zero.  Contains a workgroup barrier: every lane of the workgroup calls it.
+// A workgroup can walk kQuadChunks consecutive chunks of kQuadT quads, loading
+// chunk c + 1 before it encodes chunk c.  Measured on the 4096 x 14336 weight it
+// does not pay: 1 / 2 / 4 / 8 chunks per one-wave workgroup give 26.0 / 27.2 /
+// 29.1 / 28.6 us for NF4 - the finest grain the dispatcher can deal is the
+// fastest, as for the AdamW kernels - so the default is one chunk.
+#ifndef OA_QUAD_CHUNKS
+#define OA_QUAD_CHUNKS 1
+#endif
+constexpr int kQuadChunks = OA_QUAD_CHUNKS;
+
 template <int SRC>
-__device__ __forceinline__ void quad_fetch(const void* __restrict__ src, int64_t q0,
-                                           int64_t octets, u32x4* lds, float (&x)[4][8]) {
+struct QuadRaw {
+  u32x4 v[4][SRC == OA_F32 ? 2 : 1];
+};
+
+// Issues the loads of the chunk whose first quad is q0 (a multiple of kQuadT):
+// in trip k the lane takes octet 64 k + lane of its wave's 256.  `octets` =
+// octets of the whole matrix; lanes beyond it get zeros.
+template <int SRC>
+__device__ __forceinline__ void quad_load(const void* __restrict__ src, int64_t q0,
+                                          int64_t octets, QuadRaw<SRC>& r) {
   constexpr int P = SRC == OA_F32 ? 2 : 1;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  u32x4* mine = lds + wave * (P * 256);
   const int64_t o0 = (q0 + wave * kWave) * 4;  // first octet of this wave's chunk
-  u32x4 raw[4][P];
   const char* base = static_cast<const char*>(src) + (o0 + lane) * (16 * P);
   if ((q0 + kQuadT) * 4 <= octets) {
     // every lane of the workgroup is in range (a scalar branch): the loads carry no
@@ -315,26 +331,38 @@ __device__ __forceinline__ void quad_fetch(const void* __restrict__ src, int64_t
     for (int k = 0; k < 4; ++k)
 #pragma unroll
       for (int pl = 0; pl < P; ++pl)
-        raw[k][pl] = __builtin_nontemporal_load(
+        r.v[k][pl] = __builtin_nontemporal_load(
             reinterpret_cast<const u32x4*>(base + (int64_t)k * (64 * 16 * P)) + pl);
   } else {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const bool in = o0 + 64 * k + lane < octets;
-      // the last workgroup: out-of-range lanes re-read the matrix's first octet
+      // the matrix's last chunk: out-of-range lanes re-read its first octet
       const u32x4* p = reinterpret_cast<const u32x4*>(
           in ? base + (int64_t)k * (64 * 16 * P) : static_cast<const char*>(src));
 #pragma unroll
       for (int pl = 0; pl < P; ++pl) {
         const u32x4 v = __builtin_nontemporal_load(p + pl);
-        raw[k][pl] = in ? v : u32x4{0u, 0u, 0u, 0u};
+        r.v[k][pl] = in ? v : u32x4{0u, 0u, 0u, 0u};
       }
     }
   }
+}
+
+// Hands the loaded octets over: afterwards x holds the lane's own quad (first
+// element 32 * (q0 + threadIdx.x)).  Two workgroup barriers: every lane of the
+// workgroup calls it.
+template <int SRC>
+__device__ __forceinline__ void quad_exchange(const QuadRaw<SRC>& r, u32x4* lds,
+                                              float (&x)[4][8]) {
+  constexpr int P = SRC == OA_F32 ? 2 : 1;
+  const int lane = threadIdx.x & (kWave - 1);
+  u32x4* mine = lds + (threadIdx.x / kWave) * (P * 256);
+  __syncthreads();  // the previous chunk has been read
 #pragma unroll
   for (int k = 0; k < 4; ++k)
 #pragma unroll
-    for (int pl = 0; pl < P; ++pl) mine[pl * 256 + quad_slot(64 * k + lane)] = raw[k][pl];
+    for (int pl = 0; pl < P; ++pl) mine[pl * 256 + quad_slot(64 * k + lane)] = r.v[k][pl];
   __syncthreads();
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -543,6 +571,51 @@ dequant_int8_kernel(const int8_t* __restrict__ q, const void* __restrict__ scale
     if (i >= rows * cols) return;
     const int64_t row = i / cols, c = i - row * cols;
     store1<OUT>(out, row * ostride + c, (float)q[i] * load_scale(scales, sdt, row));
+  }
+}
+
+// The decoder's fast path with everything that made a load wait taken out: a tile
+// that lies wholly inside the matrix is a scalar condition (the last tile clamps
+// its octet index instead of guarding the load), and the scale dtype is a
+// template argument (a run-time switch puts each scale load and its convert into
+// a branch of its own).  All 2 x kOct loads of a lane are issued before the first
+// convert.  A lane owns octets, so that each store instruction of a wave covers
+// one contiguous KiB (16 codes per lane would load in one piece but store two
+// interleaved halves: measured 34 us against 31.6).
+template <int OUT, int SDT>
+__global__ void __launch_bounds__(kT)
+dequant_int8_tile_kernel(const int8_t* __restrict__ q, const void* __restrict__ scales,
+                         int64_t rows, int64_t cols, void* __restrict__ out, int64_t ostride,
+                         int mode) {
+  const int64_t opr = cols >> 3, total = rows * opr;
+  const int64_t tile0 = (int64_t)blockIdx.x * (kT * kOct);
+  const int64_t o0 = tile0 + threadIdx.x;
+  u32x2 w[kOct];
+  uint32_t sraw[kOct];
+  int64_t at[kOct];
+  const bool full = tile0 + kT * kOct <= total;
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    int64_t o = o0 + (int64_t)k * kT;
+    if (!full && o >= total) o = total - 1;  // re-read the last octet; its store is skipped
+    const int64_t row = octet_row(o, opr, mode);
+    w[k] = *reinterpret_cast<const u32x2*>(q + o * 8);
+    if (SDT == OA_F32) sraw[k] = static_cast<const uint32_t*>(scales)[row];
+    else sraw[k] = static_cast<const uint16_t*>(scales)[row];
+    at[k] = row * ostride + (o - row * opr) * 8;
+  }
+#pragma unroll
+  for (int k = 0; k < kOct; ++k) {
+    if (!full && o0 + (int64_t)k * kT >= total) continue;
+    const float sc = SDT == OA_F32 ? __uint_as_float(sraw[k])
+                     : SDT == OA_BF16 ? bf16_bits_to_f32(sraw[k]) : f16_bits_to_f32(sraw[k]);
+    float y[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int32_t v = (int32_t)(int8_t)((w[k][j >> 2] >> (8 * (j & 3))) & 0xFFu);
+      y[j] = (float)v * sc;
+    }
+    store8<OUT, false>(out, at[k], y);
   }
 }
 
@@ -932,7 +1005,7 @@ __device__ __forceinline__ uint32_t nf4_pack8r(const float (&x)[8], float inv16,
 // steps per 32 elements instead of three per octet, the correctly rounded
 // reciprocal is taken once per 32 elements, and the codes leave as one 16-byte
 // store per lane (1 KiB per wave instruction; the maxima as one run of floats).
-// The quad arrives through quad_fetch().
+// The quad arrives through quad_load() / quad_exchange().
 template <int SRC, int LPB>
 __global__ void __launch_bounds__(kQuadT)
 quant_nf4_quad_kernel(const void* __restrict__ src, int64_t quads, int lpb_arg, int lpb_shift_arg,
@@ -943,19 +1016,29 @@ quant_nf4_quad_kernel(const void* __restrict__ src, int64_t quads, int lpb_arg, 
   __shared__ u32x4 stage[quad_lds_slots<SRC>()];
   if (threadIdx.x < 64)
     lut[threadIdx.x] = u32x2{kNf4RBuckets.own16[threadIdx.x], kNf4RBuckets.below[threadIdx.x]};
-  const int64_t q0 = (int64_t)blockIdx.x * kQuadT;
-  const int64_t q = q0 + threadIdx.x;
-  float x[4][8];
-  quad_fetch<SRC>(src, q0, quads * 4, stage, x);  // its barrier also covers the table
-  float a = fmaxf(fmaxf(absmax8(x[0]), absmax8(x[1])), fmaxf(absmax8(x[2]), absmax8(x[3])));
-  a = group_max(a, lpb);
-  const float inv16 = (1.0f / fmaxf(a, kEps)) * 16.0f;
-  u32x4 w;
+  const int64_t qbase = (int64_t)blockIdx.x * (kQuadT * kQuadChunks);
+  QuadRaw<SRC> cur, nxt;
+  quad_load<SRC>(src, qbase, quads * 4, cur);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) w[j] = nf4_pack8r(x[j], inv16, lut);
-  if (q < quads) {
-    __builtin_nontemporal_store(w, packed + q);
-    if ((threadIdx.x & (lpb - 1)) == 0) absmax_out[q >> lpb_shift] = a;
+  for (int c = 0; c < kQuadChunks; ++c) {
+    const int64_t q0 = qbase + (int64_t)c * kQuadT;
+    if (q0 >= quads) break;
+    const bool more = c + 1 < kQuadChunks && q0 + kQuadT < quads;
+    if (more) quad_load<SRC>(src, q0 + kQuadT, quads * 4, nxt);
+    float x[4][8];
+    quad_exchange<SRC>(cur, stage, x);  // its barriers also cover the table
+    float a = fmaxf(fmaxf(absmax8(x[0]), absmax8(x[1])), fmaxf(absmax8(x[2]), absmax8(x[3])));
+    a = group_max(a, lpb);
+    const float inv16 = (1.0f / fmaxf(a, kEps)) * 16.0f;
+    u32x4 w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = nf4_pack8r(x[j], inv16, lut);
+    const int64_t q = q0 + threadIdx.x;
+    if (q < quads) {
+      __builtin_nontemporal_store(w, packed + q);
+      if ((threadIdx.x & (lpb - 1)) == 0) absmax_out[q >> lpb_shift] = a;
+    }
+    cur = nxt;
   }
 }
 
@@ -1120,7 +1203,10 @@ __device__ __forceinline__ float e2m1_value(uint32_t code) {
 }
 
 constexpr int kAmaxMaxBlocks = 16384;  // floats of the shared norm/amax workspace
-constexpr int kAmaxUnroll = 4;         // octets in flight per lane
+#ifndef OA_AMAX_UNROLL
+#define OA_AMAX_UNROLL 4
+#endif
+constexpr int kAmaxUnroll = OA_AMAX_UNROLL;  // octets in flight per lane
 
 // Tensor-wide max |x|, first launch: one partial maximum per block.  Octets of a
 // row-contiguous matrix are addressed flat (no per-octet division).
@@ -1283,27 +1369,37 @@ __global__ void __launch_bounds__(kQuadT)
 quant_nvfp4_quad_kernel(const void* __restrict__ src, int64_t quads, u32x4* __restrict__ packed,
                         uint16_t* __restrict__ scale16, const float* __restrict__ gs_ptr) {
   __shared__ u32x4 stage[quad_lds_slots<SRC>()];
-  const int64_t q0 = (int64_t)blockIdx.x * kQuadT;
-  const int64_t q = q0 + threadIdx.x;
-  float x[4][8];
-  quad_fetch<SRC>(src, q0, quads * 4, stage, x);
+  const int64_t qbase = (int64_t)blockIdx.x * (kQuadT * kQuadChunks);
+  QuadRaw<SRC> cur, nxt;
+  quad_load<SRC>(src, qbase, quads * 4, cur);
   const float gs = *gs_ptr;
   const float inv_global = 1.0f / gs;
-  u32x4 w;
-  uint32_t s2 = 0;
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    const float amax = fmaxf(absmax8(x[2 * b]), absmax8(x[2 * b + 1]));
-    const uint32_t s8 = nvfp4_block_scale(amax, inv_global);
-    const float eff = e4m3fn_bits_to_f32(s8) * gs;
-    const float inv_eff = 1.0f / fmaxf(eff, kEps);
-    w[2 * b] = nvfp4_pack8(x[2 * b], inv_eff);
-    w[2 * b + 1] = nvfp4_pack8(x[2 * b + 1], inv_eff);
-    s2 |= s8 << (8 * b);
-  }
-  if (q < quads) {
-    __builtin_nontemporal_store(w, packed + q);
-    scale16[q] = (uint16_t)s2;
+  for (int c = 0; c < kQuadChunks; ++c) {
+    const int64_t q0 = qbase + (int64_t)c * kQuadT;
+    if (q0 >= quads) break;
+    const bool more = c + 1 < kQuadChunks && q0 + kQuadT < quads;
+    if (more) quad_load<SRC>(src, q0 + kQuadT, quads * 4, nxt);
+    float x[4][8];
+    quad_exchange<SRC>(cur, stage, x);
+    u32x4 w;
+    uint32_t s2 = 0;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const float amax = fmaxf(absmax8(x[2 * b]), absmax8(x[2 * b + 1]));
+      const uint32_t s8 = nvfp4_block_scale(amax, inv_global);
+      const float eff = e4m3fn_bits_to_f32(s8) * gs;
+      const float inv_eff = 1.0f / fmaxf(eff, kEps);
+      w[2 * b] = nvfp4_pack8(x[2 * b], inv_eff);
+      w[2 * b + 1] = nvfp4_pack8(x[2 * b + 1], inv_eff);
+      s2 |= s8 << (8 * b);
+    }
+    const int64_t q = q0 + threadIdx.x;
+    if (q < quads) {
+      __builtin_nontemporal_store(w, packed + q);
+      scale16[q] = (uint16_t)s2;
+    }
+    cur = nxt;
   }
 }
 
@@ -1462,6 +1558,23 @@ extern "C" int oa_dequant_int8(const void* q, const void* scales, int scale_dtyp
   const int vec = rows_vec(out, out_dtype, out_row_stride, cols) && aligned_to(q, 8);
   const unsigned blocks = vec ? blocks_oct(rows * (cols / 8)) : blocks_for(rows * cols);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (vec) {
+    const int mode = div_mode(rows, cols);
+#define OA_I8_HEX(SD)                                                                        \
+  OA_DISPATCH_DT(out_dtype,                                                                  \
+                 hipLaunchKernelGGL((dequant_int8_tile_kernel<DT, SD>), dim3(blocks), dim3(kT), \
+                                    0, s, static_cast<const int8_t*>(q), scales, rows, cols,  \
+                                    out, out_row_stride, mode))
+    if (scale_dtype == OA_F32) {
+      OA_I8_HEX(OA_F32);
+    } else if (scale_dtype == OA_BF16) {
+      OA_I8_HEX(OA_BF16);
+    } else {
+      OA_I8_HEX(OA_F16);
+    }
+#undef OA_I8_HEX
+    return launch_status();
+  }
   OA_DISPATCH_DT(out_dtype,
                  hipLaunchKernelGGL(dequant_int8_kernel<DT>, dim3(blocks), dim3(kT), 0,
                                     s, static_cast<const int8_t*>(q), scales, scale_dtype, rows,
@@ -1556,7 +1669,7 @@ extern "C" int oa_quant_nf4(const void* src, int src_dtype, int64_t src_row_stri
     OA_DISPATCH_DT(src_dtype,
                    hipLaunchKernelGGL((block == 64 ? quant_nf4_quad_kernel<DT, 2>
                                                    : quant_nf4_quad_kernel<DT, 0>),
-                                      dim3((unsigned)((quads + kQuadT - 1) / kQuadT)),
+                                      dim3((unsigned)((quads + kQuadT * kQuadChunks - 1) / (kQuadT * kQuadChunks))),
                                       dim3(kQuadT), 0, s, src, quads, lpb, log2i(lpb),
                                       static_cast<u32x4*>(packed), static_cast<float*>(absmax)));
   } else if (fast) {
@@ -1638,7 +1751,7 @@ extern "C" int oa_quant_nvfp4(const void* src, int src_dtype, int64_t src_row_st
     const int64_t quads = rows * cols / 32;
     OA_DISPATCH_DT(src_dtype,
                    hipLaunchKernelGGL(quant_nvfp4_quad_kernel<DT>,
-                                      dim3((unsigned)((quads + kQuadT - 1) / kQuadT)),
+                                      dim3((unsigned)((quads + kQuadT * kQuadChunks - 1) / (kQuadT * kQuadChunks))),
                                       dim3(kQuadT), 0, s, src, quads, static_cast<u32x4*>(packed),
                                       static_cast<uint16_t*>(block_scale),
                                       static_cast<const float*>(global_scale)));
