@@ -710,16 +710,30 @@ quant_int4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, in
     }
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) encode_row(x[p], p * (kT / WPR) + rsub);
+  } else if (WPR != 0 && full) {
+    // fused AdamW source, whole tile: the loads of row pass p + 1 are issued before
+    // pass p is updated, stored and encoded (two passes of operands in registers)
+    constexpr int kRpp = kT / (WPR ? WPR : 1);
+    constexpr int kPasses = kI4RowsQ / kRpp;
+    AdamRaw raw[2];
+    float x[8];
+    fetch8_begin<SRC>(src, ad, (r0 + rsub) * stride + gi * group + k * 8, raw[0], x);
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const int64_t at = (r0 + p * kRpp + rsub) * stride + gi * group + k * 8;
+      if (p + 1 < kPasses) {
+        float unused[8];
+        fetch8_begin<SRC>(src, ad, at + (int64_t)kRpp * stride, raw[(p + 1) & 1], unused);
+      }
+      fetch8_end<SRC>(ad, at, raw[p & 1], x);
+      encode_row(x, p * kRpp + rsub);
+    }
   } else {
     for (int pr = 0; pr < kI4RowsQ; pr += rows_per_pass) {
       const int rl = pr + rsub;
       const int64_t row = r0 + rl;
       float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (full && rl < kI4RowsQ) {
-        fetch8<SRC>(src, ad, row * stride + gi * group + k * 8, x);
-      } else if (rl < kI4RowsQ && row < rows) {
-        fetch8<SRC>(src, ad, row * stride + gi * group + k * 8, x);
-      }
+      if (rl < kI4RowsQ && row < rows) fetch8<SRC>(src, ad, row * stride + gi * group + k * 8, x);
       encode_row(x, rl);
     }
   }
