@@ -419,6 +419,22 @@ __device__ __forceinline__ int32_t q_int8(float x, float inv) {
   t = fminf(fmaxf(t, -128.0f), 127.0f);
   return (int32_t)t;
 }
+// Four codes of one packed dword: clamp(rint(x * inv), -128, 127) + 128 is an
+// integer in [0, 255], exact in fp32; v_cvt_pk_u8_f32 converts it and places the
+// byte, and flipping the top bit of every byte afterwards takes the 128 off again
+// (two's complement).  A NaN clamps to -128, as in q_int8().
+__device__ __forceinline__ uint32_t q_int8_word(float a, float b, float c, float d, float inv) {
+  uint32_t w = 0;
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __builtin_amdgcn_fmed3f(__builtin_rintf(a * inv), -128.0f, 127.0f) + 128.0f, 0, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __builtin_amdgcn_fmed3f(__builtin_rintf(b * inv), -128.0f, 127.0f) + 128.0f, 1, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __builtin_amdgcn_fmed3f(__builtin_rintf(c * inv), -128.0f, 127.0f) + 128.0f, 2, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __builtin_amdgcn_fmed3f(__builtin_rintf(d * inv), -128.0f, 127.0f) + 128.0f, 3, w);
+  return w ^ 0x80808080u;
+}
 
 constexpr int kRowCache = 8;  // octets a lane keeps in registers between the two passes
 #ifndef OA_I8_BATCH
@@ -506,12 +522,8 @@ quant_int8_kernel(const void* __restrict__ src, int64_t stride, int64_t cols,
 
   int8_t* qr = q + row * cols;
   auto encode = [&](const float (&x)[8], int64_t o) {
-    uint32_t w0 = 0, w1 = 0;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      w0 |= ((uint32_t)q_int8(x[k], inv) & 0xFFu) << (8 * k);
-      w1 |= ((uint32_t)q_int8(x[4 + k], inv) & 0xFFu) << (8 * k);
-    }
+    const uint32_t w0 = q_int8_word(x[0], x[1], x[2], x[3], inv);
+    const uint32_t w1 = q_int8_word(x[4], x[5], x[6], x[7], inv);
     __builtin_nontemporal_store(u32x2{w0, w1}, reinterpret_cast<u32x2*>(qr + o * 8));
   };
   if (cached) {
@@ -621,19 +633,27 @@ dequant_int8_tile_kernel(const int8_t* __restrict__ q, const void* __restrict__ 
 
 // ------------------------------------------------------------------- int4
 
+// Eight codes of one packed word.  clamp(rint(x * inv), -8, 7) + 8 is formed in
+// fp32 (every intermediate is a small integer, hence exact), two codes are joined
+// into their byte lo + 16 hi with one multiply-add, and the byte is converted and
+// placed by one v_cvt_pk_u8_f32: 4.5 VALU operations per code instead of 7.
 __device__ __forceinline__ uint32_t q_int4_word(const float (&x)[8], float inv) {
   uint32_t word = 0;
 #pragma unroll
-  for (int k = 0; k < 8; ++k) {
-    float t = __builtin_rintf(x[k] * inv);
-    t = fminf(fmaxf(t, -8.0f), 7.0f);
-    word |= (uint32_t)((int32_t)t + 8) << (4 * k);
+  for (int k = 0; k < 4; ++k) {
+    const float lo = __builtin_amdgcn_fmed3f(__builtin_rintf(x[2 * k] * inv), -8.0f, 7.0f);
+    const float hi = __builtin_amdgcn_fmed3f(__builtin_rintf(x[2 * k + 1] * inv), -8.0f, 7.0f);
+    const float byte = __builtin_fmaf(hi, 16.0f, lo) + 136.0f;  // (hi + 8) * 16 + (lo + 8)
+    word = __builtin_amdgcn_cvt_pk_u8_f32(byte, k, word);
   }
   return word;
 }
 
-constexpr int kI4RowsQ = 64;   // rows of one LDS tile, encoder
-constexpr int kI4PitchQ = 68;  // words per LDS row of it: 16-byte aligned rows, and the
+#ifndef OA_I4_ROWS_Q
+#define OA_I4_ROWS_Q 64
+#endif
+constexpr int kI4RowsQ = OA_I4_ROWS_Q;   // rows of one LDS tile, encoder
+constexpr int kI4PitchQ = kI4RowsQ + 4;  // words per LDS row of it: 16-byte aligned rows, and the
                                // writes of a wave (16 word columns x 4 rows) hit 64 banks
 constexpr int kI4RowsD = 128;  // rows of one LDS tile, decoder
 constexpr int kI4Chunk = 4;    // decoder: packed words a lane fetches per trip
