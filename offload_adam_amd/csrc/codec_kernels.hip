@@ -1985,6 +1985,15 @@ extern "C" int oa_adam_requant_nvfp4(const void* grad, void* exp_avg, void* exp_
   rc = launch_status();
   if (rc) return rc;
   // launch 3: encode from the stored master
+  if ((rows * cols) % 32 == 0 && aligned_to(packed, 16)) {
+    const int64_t quads = rows * cols / 32;
+    hipLaunchKernelGGL(quant_nvfp4_quad_kernel<OA_F32>,
+                       dim3((unsigned)((quads + kQuadT * kQuadChunks - 1) / (kQuadT * kQuadChunks))),
+                       dim3(kQuadT), 0, s, static_cast<const void*>(master), quads,
+                       static_cast<u32x4*>(packed), static_cast<uint16_t*>(block_scale),
+                       static_cast<const float*>(global_scale));
+    return launch_status();
+  }
   hipLaunchKernelGGL(quant_nvfp4_kernel<OA_F32>, dim3(blocks_oct(octets)), dim3(kT), 0, s,
                      static_cast<const void*>(master), cols, rows, cols,
                      static_cast<uint32_t*>(packed), static_cast<uint8_t*>(block_scale),
