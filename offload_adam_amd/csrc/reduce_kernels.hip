@@ -76,7 +76,8 @@ __device__ __forceinline__ float sq8(const u32x4 w, float acc) {
 // than kMaxBlocks tiles).
 __global__ void __launch_bounds__(kThreads)
 grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, int64_t groups,
-                         float* __restrict__ partial) {
+                         float* __restrict__ partial, uint16_t* __restrict__ norm_direct,
+                         float* __restrict__ sumsq_direct) {
   __shared__ float lds[kThreads / kWave];
   const u32x4* body = reinterpret_cast<const u32x4*>(g + head);
   const int64_t tiles = (groups + kTileGroups - 1) / kTileGroups;
@@ -104,7 +105,16 @@ grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, in
   }
 
   const float total = block_sum<kThreads>(acc, lds);
-  if (threadIdx.x == 0) partial[blockIdx.x] = total;
+  if (threadIdx.x == 0) {
+    if (norm_direct) {
+      // a one-block launch is its own final pass: the second launch would add this
+      // one partial to zeros, which changes no bit
+      if (sumsq_direct) *sumsq_direct = total;
+      *norm_direct = (uint16_t)f32_to_bf16_1(sqrtf(total));
+    } else {
+      partial[blockIdx.x] = total;
+    }
+  }
 }
 
 __global__ void __launch_bounds__(kFinalThreads)
@@ -172,9 +182,13 @@ int launch_grad_norm(const void* grad, int64_t n, void* norm_out, void* sumsq_ou
   int64_t blocks = (groups + kTileGroups - 1) / kTileGroups;
   if (blocks < 1) blocks = 1;
   if (blocks > kMaxBlocks) blocks = kMaxBlocks;
+  const bool single = blocks == 1;  // tensors of up to 16384 elements: one launch, not two
   hipLaunchKernelGGL(grad_norm_partial_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, s,
-                     static_cast<const uint16_t*>(grad), n, (int)head, groups, partial);
+                     static_cast<const uint16_t*>(grad), n, (int)head, groups, partial,
+                     single ? static_cast<uint16_t*>(norm_out) : nullptr,
+                     single ? static_cast<float*>(sumsq_out) : nullptr);
   int rc = launch_status();
+  if (single) return rc;
   if (rc) return rc;
   hipLaunchKernelGGL(grad_norm_final_kernel, dim3(1), dim3(kFinalThreads), 0, s, partial,
                      (int)blocks, static_cast<uint16_t*>(norm_out),
