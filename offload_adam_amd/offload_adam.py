@@ -22,6 +22,7 @@ What runs underneath is this package's HIP library: the fused AdamW kernels
 """
 
 import bisect
+import sys
 import time
 import warnings
 from ctypes import c_int, c_size_t, c_void_p
@@ -444,10 +445,12 @@ class OffloadAdam(Optimizer):
             cached_s = sum(p.numel() for p in self._state_cached) * (
                 sum(torch.empty(0, dtype=d).element_size()
                     for k, d in self.offload_config.items() if k != "grad"))
+            # part of the verbose report on stdout; at verbose=0 (spare_hbm) a notice on stderr
             print(f"HBM the optimizer may hold: gradient cache {cached_g / _GIB:.2f} GB "
                   f"({len(self._grad_cached)} params), state cache {cached_s / _GIB:.2f} GB "
                   f"({len(self._state_cached)} params), prefetch staging "
-                  f"{self._PREFETCH_BYTES / _GIB:.2f} GB")
+                  f"{self._PREFETCH_BYTES / _GIB:.2f} GB",
+                  file=sys.stdout if self.verbose > 0 else sys.stderr)
 
         self._pending_steps = []      # offloaded parameters waiting for their group's launch
         self._pending_inplace = []    # GPU-resident ones

@@ -928,8 +928,8 @@ def test_default_contract_is_the_reference_one(fixed_seed, capsys):
             assert opt.device_states[p].get("grad") is None  # nothing kept in HBM
 
     model, opt = build(spare_hbm=True)
-    out = capsys.readouterr().out
-    assert "HBM the optimizer may hold" in out
+    captured = capsys.readouterr()
+    assert captured.out == "" and "HBM the optimizer may hold" in captured.err
     assert opt._grad_cache_write_back and len(opt._grad_cached) == len(opt._offload_params)
     assert len(opt._state_cached) == len(opt._offload_params)
     with pytest.raises(ValueError, match="prefetch_bytes"):
