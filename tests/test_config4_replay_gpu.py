@@ -10,9 +10,12 @@ hook consumes it, the bf16 accumulation (src/offload_adam/offload_adam.py:398,
 528) is redone with CPU tensors, ``oracle.adam_stochastic_rounding`` is applied
 with the seeds the optimizer drew, and parameters and both moments must be
 bit-equal after each of three steps.  ``Adam`` (states in HBM, plain ``step()``)
-is checked the same way.
+is checked the same way, and so are the other three modes on the hook path and
+benchmark config 2 in the small: the clipping path (gradient norms recorded in the
+hooks, global coefficient and fused clip in ``step()``).
 """
 
+import ctypes
 import sys
 import warnings
 from pathlib import Path
@@ -68,28 +71,48 @@ class SeedLog:
         return self.real(mode, params, states, *args, **kw)
 
 
-class OracleReplica:
-    """CPU copy of parameters and moments, advanced by the oracle."""
+AUX_KEY = {"stochastic_rounding": None, "fp32_master": "master_params",
+           "fp31_master": "rounding_error", "fp32_master_custom_rounding": "rounding_error"}
 
-    def __init__(self, oracle, model, decoupled):
-        self.oracle, self.decoupled = oracle, decoupled
+
+class OracleReplica:
+    """CPU copy of parameters, moments and the mode's extra state, advanced by the oracle."""
+
+    def __init__(self, oracle, model, decoupled, mode="stochastic_rounding"):
+        self.oracle, self.decoupled, self.mode = oracle, decoupled, mode
         self.names = [n for n, _ in model.named_parameters()]
         self.p = {n: u16(p) for n, p in model.named_parameters()}
         self.m = {n: np.zeros_like(b) for n, b in self.p.items()}
         self.v = {n: np.zeros_like(b) for n, b in self.p.items()}
+        if mode == "fp32_master":  # the master starts as the widened parameter
+            self.aux = {n: p.detach().float().cpu().numpy().reshape(-1).copy()
+                        for n, p in model.named_parameters()}
+        elif AUX_KEY[mode]:
+            self.aux = {n: np.zeros(b.size, dtype=np.int16) for n, b in self.p.items()}
         self.step = 0
 
-    def advance(self, grads, seeds, layout):
-        """``grads[name]``: the micro-batch gradients in firing order (CPU bf16)."""
+    def total_gradient(self, grads, n):
+        total = grads[n][0].clone()
+        for g in grads[n][1:]:
+            total.add_(g)  # bf16 += bf16: fp32 sum, one rounding, as on the GPU
+        return u16(total)
+
+    def advance(self, grads, seeds=None, layout=0, clip=None):
+        """``grads[name]``: the micro-batch gradients in firing order (CPU bf16);
+        ``clip``: bf16 bits of the clip coefficient or None."""
         self.step += 1
         b1h, b2h = self.oracle.folded_betas(*HYP["betas"], self.step)
+        hyp = (HYP["lr"], HYP["weight_decay"], b1h, b2h, HYP["eps"], self.decoupled)
         for n in self.names:
-            total = grads[n][0].clone()
-            for g in grads[n][1:]:
-                total.add_(g)  # bf16 += bf16: fp32 sum, one rounding, as on the GPU
-            self.oracle.adam_stochastic_rounding(
-                self.p[n], u16(total), self.m[n], self.v[n], HYP["lr"], HYP["weight_decay"],
-                b1h, b2h, HYP["eps"], self.decoupled, seed=seeds[n], layout=layout)
+            g = self.total_gradient(grads, n)
+            if self.mode == "stochastic_rounding":
+                self.oracle.adam_stochastic_rounding(self.p[n], g, self.m[n], self.v[n], *hyp,
+                                                     seed=seeds[n], layout=layout, clip=clip)
+            else:
+                fn = {"fp32_master": self.oracle.adam_fp32_master,
+                      "fp31_master": self.oracle.adam_fp31_master,
+                      "fp32_master_custom_rounding": self.oracle.adam_custom_rounding}[self.mode]
+                fn(self.p[n], g, self.m[n], self.v[n], self.aux[n], *hyp, clip=clip)
 
     def assert_equal(self, model, state_of, step):
         for n, p in model.named_parameters():
@@ -97,6 +120,14 @@ class OracleReplica:
             assert np.array_equal(u16(p), self.p[n]), f"step {step}: param {n}"
             assert np.array_equal(u16(st["exp_avg"]), self.m[n]), f"step {step}: exp_avg {n}"
             assert np.array_equal(u16(st["exp_avg_sq"]), self.v[n]), f"step {step}: exp_avg_sq {n}"
+            key = AUX_KEY[self.mode]
+            if key == "master_params":
+                got = st[key].detach().cpu().numpy().reshape(-1)
+                assert np.array_equal(got.view(np.uint32), self.aux[n].view(np.uint32)), \
+                    f"step {step}: master {n}"
+            elif key:
+                got = st[key].detach().cpu().numpy().reshape(-1)
+                assert np.array_equal(got, self.aux[n]), f"step {step}: rounding_error {n}"
 
 
 def capture_hooks(model, sink):
@@ -190,4 +221,102 @@ def test_resident_adam_equals_the_oracle(oracle, monkeypatch, rng):
         seeds = {ptr_name[ptr]: seed for ptr, seed in log.by_ptr.items()}
         assert len(seeds) == len(ptr_name)
         replica.advance(per_mb, seeds, LAYOUT[rng])
+        replica.assert_equal(model, lambda p: opt.state[p], s + 1)
+
+
+@pytest.mark.parametrize("mode", ["fp32_master", "fp31_master", "fp32_master_custom_rounding"])
+@pytest.mark.parametrize("caches", sorted(CACHES))
+def test_offload_adam_other_modes_equal_the_oracle(oracle, mode, caches):
+    from offload_adam_amd import OffloadAdam
+
+    model = tiny_decoder()
+    replica = OracleReplica(oracle, model, True, mode)
+    grads = {}
+    capture_hooks(model, grads)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode=mode, inplace_param_threshold=THRESHOLD,
+                          decoupled_weight_decay=True, **HYP, **CACHES[caches])
+    data = token_batches(model.c["vocab"])
+    for s in range(STEPS):
+        grads.clear()
+        for mb in range(GA):
+            opt.ready_for_optimizer_step = mb == GA - 1
+            model(data[s * GA + mb]).backward()
+        opt.step()
+        opt.zero_grad()
+        torch.cuda.synchronize()
+        replica.advance(grads)
+        replica.assert_equal(model, lambda p: opt.state[p], s + 1)
+
+
+@pytest.mark.parametrize("mode", ["fp31_master", "stochastic_rounding"])
+@pytest.mark.parametrize("caches", sorted(CACHES))
+def test_clipping_path_equals_the_oracle(oracle, monkeypatch, mode, caches):
+    """Benchmark config 2 in the small (src/offload_adam/offload_adam.py:504-505,
+    542-571): per-parameter norms from the hooks within one bf16 ulp of the oracle's,
+    the global norm and the coefficient bit-equal given those norms, and the clipped
+    update bit-equal."""
+    from offload_adam_amd import OffloadAdam
+    from offload_adam_amd import offload_adam as oa_mod
+    from offload_adam_amd.kernels import stochastic_rounding as sr_mod
+
+    max_norm = 0.25
+    seeds_by_ptr = {}
+    if mode == "stochastic_rounding":
+        # the clipping path steps parameter by parameter through the single-tensor entry
+        real = sr_mod.adam_step_stochastic_rounding
+        counter = [0]
+
+        def logged(params, states, *args, **kw):
+            counter[0] += 1
+            seed = (0x9E3779B97F4A7C15 * counter[0] + 99) & 0xFFFFFFFFFFFFFFFF
+            seeds_by_ptr[params.data_ptr()] = seed
+            kw.update(seed=seed, rng="triton")
+            return real(params, states, *args, **kw)
+
+        monkeypatch.setitem(oa_mod.OffloadAdam.supported_modes[mode], "step", logged)
+        log = SeedLog(oa_mod.adam_step_multi, "triton")  # the GPU-resident small parameters
+        monkeypatch.setattr(oa_mod, "adam_step_multi", log)
+    model = tiny_decoder()
+    replica = OracleReplica(oracle, model, True, mode)
+    grads = {}
+    capture_hooks(model, grads)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = OffloadAdam(model, mode=mode, max_grad_norm=max_norm,
+                          inplace_param_threshold=THRESHOLD, decoupled_weight_decay=True,
+                          **HYP, **CACHES[caches])
+    names = {p: n for n, p in model.named_parameters()}
+    order = [names[p] for g in opt.param_groups for p in g["params"]]
+    ptr_name = {p.data_ptr(): n for n, p in model.named_parameters()}
+    data = token_batches(model.c["vocab"])
+    for s in range(STEPS):
+        grads.clear()
+        seeds_by_ptr.clear()
+        if mode == "stochastic_rounding":
+            log.by_ptr.clear()
+        for mb in range(GA):
+            opt.ready_for_optimizer_step = mb == GA - 1
+            model(data[s * GA + mb]).backward()
+        opt.step()
+        opt.zero_grad()
+        torch.cuda.synchronize()
+        gpu_norms = u16(opt._norm_slots)
+        for i, n in enumerate(order):
+            want = int(oracle.grad_norm_bf16(replica.total_gradient(grads, n)))
+            assert abs(int(gpu_norms[i]) - want) <= 1, (s, n, gpu_norms[i], want)
+        total = oracle.lib().oaref_total_norm_bf16(
+            gpu_norms.ctypes.data_as(ctypes.c_void_p), len(order))
+        assert int(u16(opt._total_norm.reshape(1))[0]) == total
+        coef = oracle.clip_coef_bf16(total, max_norm)
+        assert int(u16(opt._clip_coef.reshape(1))[0]) == coef
+        assert coef < 0x3F80, "the threshold must clip"
+        seeds = None
+        if mode == "stochastic_rounding":
+            merged = dict(seeds_by_ptr)
+            merged.update(log.by_ptr)
+            seeds = {ptr_name[ptr]: seed for ptr, seed in merged.items()}
+            assert len(seeds) == len(ptr_name)
+        replica.advance(grads, seeds, LAYOUT["triton"], clip=coef)
         replica.assert_equal(model, lambda p: opt.state[p], s + 1)
