@@ -72,9 +72,23 @@ __device__ __forceinline__ void adam_core(float& M, float g, float& m, float& v,
 
 // Philox4x32-10 (Salmon et al., SC'11): round multipliers 0xD2511F53 and
 // 0xCD9E8D57, key increments 0x9E3779B9 and 0xBB67AE85.
+#ifndef OA_PHILOX_XOR3
+#define OA_PHILOX_XOR3 1
+#endif
 struct Philox {
   uint32_t c0, c1, c2, c3;
 };
+
+// a ^ b ^ c in one instruction (gfx950's three-input bit operation with the
+// truth table of a three-way xor); the compiler leaves two v_xor_b32 otherwise,
+// and with one Philox block per element the update is bound by instruction issue.
+__device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
+#if OA_PHILOX_XOR3
+  return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+#else
+  return a ^ b ^ c;
+#endif
+}
 
 __device__ __forceinline__ Philox philox4x32_10(uint32_t c0, uint32_t c1,
                                                 uint32_t c2, uint32_t c3,
@@ -83,8 +97,9 @@ __device__ __forceinline__ Philox philox4x32_10(uint32_t c0, uint32_t c1,
   for (int r = 0; r < 10; ++r) {
     const uint64_t pb = (uint64_t)0xCD9E8D57u * (uint64_t)c2;
     const uint64_t pa = (uint64_t)0xD2511F53u * (uint64_t)c0;
-    const uint32_t n0 = (uint32_t)(pb >> 32) ^ c1 ^ k0;
-    const uint32_t n2 = (uint32_t)(pa >> 32) ^ c3 ^ k1;
+    // the first round sees the constant words of the counter: plain xors fold away
+    const uint32_t n0 = r == 0 ? (uint32_t)(pb >> 32) ^ c1 ^ k0 : xor3((uint32_t)(pb >> 32), c1, k0);
+    const uint32_t n2 = r == 0 ? (uint32_t)(pa >> 32) ^ c3 ^ k1 : xor3((uint32_t)(pa >> 32), c3, k1);
     c1 = (uint32_t)pb;
     c3 = (uint32_t)pa;
     c0 = n0;
