@@ -1068,8 +1068,10 @@ def test_transfer_streams_are_picked_by_measured_concurrency():
         warnings.simplefilter("error")  # a failed search warns
         h2d, d2h, report = pick_transfer_streams(torch.device("cuda:0"))
     assert h2d.cuda_stream != d2h.cuda_stream
-    assert report["concurrent"] and report["duplex_ratio"] < 0.85, report
-    assert report["with_compute_ratio"] < 0.85, report
+    # serialised work measures 1.0; copies that overlap measure 0.6 (two directions)
+    # and 0.72 (beside a kernel) on an idle MI355X
+    assert report["concurrent"] and report["duplex_ratio"] < 0.9, report
+    assert report["with_compute_ratio"] < 0.9, report
     _, opt = run_offload_adam("stochastic_rounding", steps=1, ga=1)
     assert opt.transfer_stream_report["concurrent"], opt.transfer_stream_report
 
