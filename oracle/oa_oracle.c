@@ -12,6 +12,8 @@
  *
  * What pins each function (tests/test_oracle_*.py):
  *   philox4x32_10          Random123 known-answer vectors
+ *   triton_randint         the words of Triton 3.6.0's own tl.randint (run by its CPU
+ *                          interpreter; tests/golden/triton_randint.npz)
  *   sr_round               exhaustive over the 65536 low halves x edge draws
  *   fp31 / custom split    brute force over all low halves, round-trip identities
  *   adam_*                 closed forms (t=1), fp64 evaluation (<= 1 ulp),

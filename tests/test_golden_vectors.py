@@ -318,3 +318,53 @@ def test_hip_codecs_equal_reference_fixtures(fmt):
                 assert np.array_equal(raw_bits(ops.dequantize_nvfp4(packed, s8, gs, cols, dt)),
                                       fx(case, f"dequant_{short}")), (case, short)
         del sdt
+
+
+# ----------------------------------------------- Triton's own tl.randint words
+#
+# tests/golden/triton_randint.npz was written by Triton 3.6.0's interpreter on
+# the CPU (tests/golden/make_triton_randint_fixture.py): the third-party code the
+# reference calls at src/offload_adam/kernels/stochastic_rounding.py:77, not a
+# restatement of it.
+
+TRITON_WORDS = np.load(Path(__file__).parent / "golden" / "triton_randint.npz")
+
+
+def test_oracle_randint_equals_tritons_own(oracle):
+    lib = oracle.lib()
+    seeds = [int(s) for s in TRITON_WORDS["seeds"]]
+    far = [int(o) for o in TRITON_WORDS["far_offsets"]]
+    assert len(seeds) == 6 and max(far) == (1 << 31) - 1
+    for i, seed in enumerate(seeds):
+        want = TRITON_WORDS[f"seed{i}_first4096"]
+        got = np.array([lib.oaref_triton_randint(seed, o) for o in range(4096)], dtype=np.uint32)
+        assert np.array_equal(got, want), hex(seed)
+        # the 16 bits the update uses, through the array form the parity tests call
+        assert np.array_equal(oracle.rand16_array(seed, 4096, 0), (want & 0xFFFF).astype(np.uint16))
+        got_far = np.array([lib.oaref_triton_randint(seed, o) for o in far], dtype=np.uint32)
+        assert np.array_equal(got_far, TRITON_WORDS[f"seed{i}_far"]), hex(seed)
+
+
+@pytest.mark.gpu
+def test_hip_reference_layout_uses_tritons_words():
+    """The kernel's reference bit layout against the same kernel fed Triton's words
+    as a buffer: identical parameters for every seed of the fixture."""
+    from offload_adam_amd.kernels import adam_step_stochastic_rounding
+
+    n = 4096
+    g = torch.Generator().manual_seed(11)
+    p0 = (torch.randn(n, generator=g) * 0.02).to(torch.bfloat16).cuda()
+    st0 = {"grad": (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16).cuda(),
+           "exp_avg": (torch.randn(n, generator=g) * 1e-4).to(torch.bfloat16).cuda(),
+           "exp_avg_sq": (torch.randn(n, generator=g) * 1e-3).square().to(torch.bfloat16).cuda()}
+    hyp = (1e-2, 0.01, 0.9, 0.999, 1e-8, 3)
+    for i, seed in enumerate(int(s) for s in TRITON_WORDS["seeds"]):
+        bits = (TRITON_WORDS[f"seed{i}_first4096"] & 0xFFFF).astype(np.uint16).view(np.int16)
+        rand16 = torch.from_numpy(bits.copy()).cuda()
+        pa, pb = p0.clone(), p0.clone()
+        sa = {k: v.clone() for k, v in st0.items()}
+        sb = {k: v.clone() for k, v in st0.items()}
+        adam_step_stochastic_rounding(pa, sa, *hyp, seed=seed, rng="triton")
+        adam_step_stochastic_rounding(pb, sb, *hyp, seed=0, rng="buffer", rand16=rand16)
+        assert torch.equal(pa.view(torch.int16), pb.view(torch.int16)), hex(seed)
+        assert not torch.equal(pa.view(torch.int16), p0.view(torch.int16))
