@@ -519,6 +519,7 @@ def run_e2e(extra, steps, warmup, timeout_s):
             "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak", "link_floor_s", "pinned_GiB",
             "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB",
             "peak_gpu_GiB", "optimizer_init_s", "copy_engines", "transfer_streams", "check",
+            "max_grad_norm",
             "loss_finite")
     row = {k: full[k] for k in keep if k in full}
     peak = (full.get("link_peak") or {}).get("bidir_each_GBps")
@@ -539,13 +540,18 @@ def offloaded_step_8b():
       reference's traffic and memory contract - followed by a numerical check of
       one more step;
     * ``spare_hbm``: ``OffloadAdam(spare_hbm=True)``;
-    * ``resident_adam``: the same loop with the GPU-resident ``Adam`` for scale."""
+    * ``resident_adam``: the same loop with the GPU-resident ``Adam`` for scale;
+    * ``clip_path_fp31``: benchmark config 2 as a training step on the same model -
+      ``fp31_master``, ``max_grad_norm=1.0`` (norms in the hooks, one-shot ``step()``),
+      default memory contract - with the numerical check of one more step."""
     return {
         "model": "llama8b (32 layers, hidden 4096, vocab 128256), bf16, 1 x 4096 tokens x 4 "
                  "micro-batches, activation checkpointing",
         "reference_traffic": run_e2e(["--check"], steps=5, warmup=2, timeout_s=300),
         "spare_hbm": run_e2e(["--spare-hbm"], steps=8, warmup=2, timeout_s=300),
         "resident_adam": run_e2e(["--optimizer", "adam"], steps=4, warmup=1, timeout_s=300),
+        "clip_path_fp31": run_e2e(["--mode", "fp31_master", "--max-grad-norm", "1.0", "--check"],
+                                  steps=3, warmup=1, timeout_s=300),
     }
 
 
@@ -569,7 +575,7 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip configs 0, 2 and 3 (about half a minute)")
     ap.add_argument("--no-e2e", action="store_true",
-                    help="skip the 8B training steps (bench_e2e.py, three child processes after "
+                    help="skip the 8B training steps (bench_e2e.py, four child processes after "
                          "the timed region; two to three minutes)")
     ap.add_argument("--no-events", action="store_true",
                     help="skip per-launch HIP events (used for profiler runs)")

@@ -297,7 +297,17 @@ class StepCheck:
     of the micro-batch gradients), every parameter on one of the two bf16
     neighbours of the fp32 result (taken within 1 fp32 ulp: torch's sqrt and
     divide are not promised correctly rounded), and the number of round-ups equal
-    to the sum of the round-up probabilities within 6 standard deviations."""
+    to the sum of the round-up probabilities within 6 standard deviations.
+
+    With ``fp31_master`` (benchmark config 2 as a training step, with or without
+    the clipping path) the gradient is first scaled as ``grad.mul_(clip_coef)``
+    would, the moments are again exact, and the master the optimizer left behind
+    - the parameter's bf16 bits plus twice its int16 rounding error - must be the
+    31-bit rounding of the fp32 result (same 1-ulp allowance), with the parameter
+    its bf16 rounding.  Every sampled per-parameter norm must lie within one bf16
+    ulp of the fp64 norm of the summed gradient, the total within one of the
+    norm of all the slots, and the coefficient must equal the reference's bf16
+    expression ``clamp(max_norm / (total + 1e-6), max=1.0)`` bit for bit."""
 
     def __init__(self, torch, model):
         self.torch, self.armed, self.grads, self.sample = torch, False, {}, {}
@@ -318,8 +328,42 @@ class StepCheck:
         self.old = {p: (p.detach().clone(), opt.state[p]["exp_avg"].to(p.device, copy=True),
                         opt.state[p]["exp_avg_sq"].to(p.device, copy=True))
                     for p in self.sample}
+        self.old_err = {p: opt.state[p]["rounding_error"].to(p.device, copy=True)
+                        for p in self.sample if "rounding_error" in opt.state[p]}
         self.grads.clear()
         self.armed = True
+
+    @staticmethod
+    def _bf16_neighbours(torch, got_bf16, exact_f64):
+        """True where the bf16 value is the exact one rounded down or up."""
+        near = exact_f64.to(torch.float32).to(torch.bfloat16)
+        bits = near.view(torch.int16).to(torch.int32)
+        got = got_bf16.view(torch.int16).to(torch.int32)
+        return (got - bits).abs() <= 1
+
+    def _check_clipping(self, opt, totals, report):
+        """Norm slots, total norm and coefficient of the clipping path."""
+        torch = self.torch
+        ok = True
+        for p, name in self.sample.items():
+            exact = totals[p].double().square().sum().sqrt()
+            if not bool(self._bf16_neighbours(torch, opt.state[p]["grad_norm"].reshape(1),
+                                              exact.reshape(1)).all()):
+                ok = False
+                report["failed"].append(name + ": gradient norm")
+        exact_total = opt._norm_slots.double().square().sum().sqrt()
+        if not bool(self._bf16_neighbours(torch, opt._total_norm.reshape(1),
+                                          exact_total.reshape(1)).all()):
+            ok = False
+            report["failed"].append("total norm")
+        want = torch.clamp(float(opt.max_grad_norm) / (opt._total_norm + 1e-6), max=1.0)
+        if not torch.equal(want.view(torch.int16), opt._clip_coef.view(torch.int16)):
+            ok = False
+            report["failed"].append("clip coefficient")
+        report["norms_within_1_bf16_ulp_and_coef_exact"] = ok
+        report["total_norm"] = float(opt._total_norm)
+        report["clip_coef"] = float(opt._clip_coef)
+        return ok
 
     def after(self, opt, decoupled):
         import numpy as np
@@ -329,6 +373,8 @@ class StepCheck:
         torch = self.torch
         self.armed = False
         torch.cuda.synchronize()
+        if opt.mode == "fp31_master":
+            return self._after_fp31(opt)
         f32 = np.float32
         group = opt.param_groups[0]
         lr, eps, wd = float(f32(group["lr"])), float(f32(group["eps"])), group["weight_decay"]
@@ -383,6 +429,76 @@ class StepCheck:
                             and report["unbiased_within_6_sigma"])
         return report
 
+    def _after_fp31(self, opt):
+        import numpy as np
+
+        torch = self.torch
+        f32 = np.float32
+        group = opt.param_groups[0]
+        lr, eps, wd = float(f32(group["lr"])), float(f32(group["eps"])), group["weight_decay"]
+        lr_wd = float(f32(group["lr"]) * f32(wd))
+        beta1, beta2 = group["betas"]
+        report = {"tensors": len(self.sample), "elements": 0, "moments_exact": True,
+                  "master_is_fp31_of_the_fp32_result": True, "param_is_bf16_of_the_master": True,
+                  "failed": []}
+        totals = {}
+        for p in self.sample:
+            total = self.grads[p][0]
+            for g in self.grads[p][1:]:
+                total.add_(g)  # bf16 += bf16, as the optimizer accumulates
+            totals[p] = total
+        clipped_ok = True
+        coef = None
+        if opt.max_grad_norm is not None:
+            clipped_ok = self._check_clipping(opt, totals, report)
+            coef = opt._clip_coef.float()
+
+        def round31(bits):
+            up = bits & (bits >> 1) & 1
+            return ((bits >> 1) + up) << 1
+
+        for p, name in self.sample.items():
+            step = opt.state[p]["step"]
+            b1h = (beta1**step - beta1) / (beta1**step - 1)
+            b2h = (beta2**step - beta2) / (beta2**step - 1)
+            omb1, omb2 = float(f32(1) - f32(b1h)), float(f32(1) - f32(b2h))
+            p0, m0, v0 = self.old.pop(p)
+            err0 = self.old_err.pop(p).to(torch.int32)
+            g = totals.pop(p).float()
+            if coef is not None:
+                g = (g * coef).to(torch.bfloat16).float()  # grad.mul_(clip_coef) in bf16
+            m0, v0 = m0.float(), v0.float()
+            m = m0 + omb1 * (g - m0)
+            v = v0 + omb2 * (g * g - v0)
+            m_now = opt.state[p]["exp_avg"].to(p.device)
+            v_now = opt.state[p]["exp_avg_sq"].to(p.device)
+            if not (torch.equal(m_now, m.to(torch.bfloat16))
+                    and torch.equal(v_now, v.to(torch.bfloat16))):
+                report["moments_exact"] = False
+                report["failed"].append(name + ": moments")
+            M0 = ((p0.view(torch.int16).to(torch.int32) << 16) + (err0 << 1)).view(torch.float32)
+            M = M0 - lr_wd * M0
+            M = M - (lr * m) / (torch.sqrt(v) + eps)
+            mb = M.view(torch.int32)
+            err_now = opt.state[p]["rounding_error"].to(p.device).to(torch.int32)
+            pb = p.detach().view(torch.int16).to(torch.int32) << 16
+            master_now = pb + (err_now << 1)
+            ok = ((master_now == round31(mb)) | (master_now == round31(mb + 1))
+                  | (master_now == round31(mb - 1)))
+            if not bool(ok.all()) or int(err_now.abs().max()) > 16384:
+                report["master_is_fp31_of_the_fp32_result"] = False
+                report["failed"].append(f"{name}: {int((~ok).sum())} masters off")
+            if not torch.equal(master_now.view(torch.float32).to(torch.bfloat16).view(torch.int16),
+                               p.detach().view(torch.int16)):
+                report["param_is_bf16_of_the_master"] = False
+                report["failed"].append(name + ": param is not the bf16 rounding of its master")
+            report["elements"] += p.numel()
+            del p0, m0, v0, err0, g, m, v, M0, M, mb, err_now, pb, master_now, ok
+        self.grads.clear()
+        report["passed"] = (report["moments_exact"] and report["master_is_fp31_of_the_fp32_result"]
+                            and report["param_is_bf16_of_the_master"] and clipped_ok)
+        return report
+
 
 def run(args):
     import torch
@@ -420,8 +536,11 @@ def run(args):
 
     check = None
     if args.check:
-        if args.mode != "stochastic_rounding" or args.max_grad_norm is not None or args.qat:
-            raise SystemExit("--check covers the stochastic-rounding hook path (config 4)")
+        if args.qat or not (
+                (args.mode == "stochastic_rounding" and args.max_grad_norm is None)
+                or args.mode == "fp31_master"):
+            raise SystemExit("--check covers the stochastic-rounding hook path (config 4) and "
+                             "fp31_master with or without clipping (config 2)")
         check = StepCheck(torch, model)  # its hooks must precede the optimizer's
 
     compute_done = {}

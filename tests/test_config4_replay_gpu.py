@@ -320,3 +320,46 @@ def test_clipping_path_equals_the_oracle(oracle, monkeypatch, mode, caches):
             assert len(seeds) == len(ptr_name)
         replica.advance(grads, seeds, LAYOUT["triton"], clip=coef)
         replica.assert_equal(model, lambda p: opt.state[p], s + 1)
+
+
+@pytest.mark.parametrize("mode,max_norm", [("stochastic_rounding", None), ("fp31_master", None),
+                                           ("fp31_master", 0.25)])
+def test_the_benchmarks_own_step_check_passes_and_can_fail(mode, max_norm):
+    """``bench_e2e.py --check`` (what vouches for the 8B runs of the bench line) on the
+    tiny decoder: it passes on an honest step and fails when one moment is off by a bit."""
+    import bench_e2e
+    from offload_adam_amd import OffloadAdam
+
+    results = []
+    for tamper in (False, True):
+        torch.manual_seed(0)
+        model = tiny_decoder()
+        check = bench_e2e.StepCheck(torch, model)  # its hooks precede the optimizer's
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            opt = OffloadAdam(model, mode=mode, max_grad_norm=max_norm, lr=1e-3, weight_decay=0.1,
+                              decoupled_weight_decay=True, inplace_param_threshold=THRESHOLD)
+        data = token_batches(model.c["vocab"])
+
+        def one_step(s):
+            for mb in range(GA):
+                opt.ready_for_optimizer_step = mb == GA - 1
+                model(data[s * GA + mb]).backward()
+            opt.step()
+            opt.zero_grad()
+
+        one_step(0)
+        check.before(opt)
+        one_step(1)
+        torch.cuda.synchronize()
+        if tamper:
+            p = next(iter(check.sample))
+            st = opt.state[p]["exp_avg"]
+            st.view(torch.int16).reshape(-1)[7] ^= 1
+        results.append(check.after(opt, decoupled=True))
+    honest, tampered = results
+    assert honest["passed"] and honest["failed"] == [], honest
+    assert honest["elements"] > 500_000
+    if max_norm is not None:
+        assert honest["clip_coef"] < 1.0 and honest["norms_within_1_bf16_ulp_and_coef_exact"]
+    assert not tampered["passed"] and not tampered["moments_exact"], tampered
