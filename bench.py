@@ -19,7 +19,10 @@ After the timed region of the default workload the same line also carries
   a small ``cpu_baseline``;
 * ``offloaded_step_8b``: config 4 as a training step through ``OffloadAdam``
   (child processes running bench_e2e.py): at the reference's traffic, with the
-  HBM caches, and the same model with the GPU-resident ``Adam``.
+  HBM caches, the same model with the GPU-resident ``Adam``, and config 2 as a
+  training step (fp31_master with the clipping path);
+* ``offloaded_step_1b``: config 1 as a training step (the 1.1B set streamed, one
+  micro-batch per step).
 
 ``--only-main`` stops after the timed region.  Only one GPU is used;
 ``--gpus N`` with N > 1 exits with a message.
@@ -499,10 +502,10 @@ def other_configs(cpu=True):
     return out
 
 
-def run_e2e(extra, steps, warmup, timeout_s):
+def run_e2e(extra, steps, warmup, timeout_s, model="llama8b"):
     import subprocess
 
-    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", "llama8b", "--steps", str(steps),
+    cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", model, "--steps", str(steps),
            "--warmup", str(warmup)] + extra
     try:
         res = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout_s, cwd=str(ROOT))
@@ -651,6 +654,10 @@ def main():
             out["other_configs"] = other_configs(cpu=not args.no_cpu_baseline)
         if not args.no_e2e:
             out["offloaded_step_8b"] = offloaded_step_8b()
+            # benchmark config 1 as a training step: the 1.1B set streamed through the
+            # default OffloadAdam, one micro-batch of 4096 tokens per step, with the check
+            out["offloaded_step_1b"] = run_e2e(["--grad-accum", "1", "--check"], steps=10,
+                                               warmup=3, timeout_s=200, model="llama1b")
     print(json.dumps(out))
 
 
