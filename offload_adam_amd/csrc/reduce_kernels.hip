@@ -98,7 +98,8 @@ grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, in
     const int64_t tail_start = head + groups * 8;
     const int64_t extra = head + (n - tail_start);  // < 16
     if (threadIdx.x < extra) {
-      const int64_t idx = threadIdx.x < head ? threadIdx.x : tail_start + (threadIdx.x - head);
+      const int64_t t = threadIdx.x;
+      const int64_t idx = t < head ? t : tail_start + (t - head);
       const float x = bf16_bits_to_f32(g[idx]);
       acc = fmaf(x, x, acc);
     }
