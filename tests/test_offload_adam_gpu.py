@@ -901,7 +901,9 @@ def test_default_contract_is_the_reference_one(fixed_seed, capsys):
     model, opt = build()
     assert capsys.readouterr().out == ""
     assert not opt._grad_cached and not opt._state_cached and not opt._grad_cache_write_back
-    assert opt._PREFETCH_BYTES == 4 << 30 and opt._prestage_bytes == 4 << 30
+    # a bounded staging window: 4 GiB, or an eighth of what is offloaded (at least 256 MiB)
+    assert opt._PREFETCH_BYTES == 256 << 20 and opt._prestage_bytes == 256 << 20
+    assert OffloadAdam._PREFETCH_BYTES == 4 << 30
     names = {p: n for n, p in model.named_parameters()}
     sums = {}
 
