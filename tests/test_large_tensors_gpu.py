@@ -176,7 +176,8 @@ def big_weight():
     torch.cuda.empty_cache()
 
 
-WINDOWS = ((0, 8), (32760, 32776), (16380, 16392))  # first, last, and around element 2^30 * 65536 / 65536
+# rows: the first; the last, which straddle element 2^31 (row 32768); those around element 2^30
+WINDOWS = ((0, 8), (32760, 32776), (16380, 16392))
 
 
 def rows_f32(w, lo, hi):
@@ -259,3 +260,51 @@ def test_nvfp4_codec_on_more_than_2_31_elements(oracle, big_weight):
         want_back = oracle.dequant_nvfp4(got_p, got_s, want_gs).reshape(-1)
         assert np.array_equal(u16(back[lo:hi]), want_back), lo
         first = False
+
+
+@pytest.mark.parametrize("fmt", ["int8", "int4", "nf4", "nvfp4"])
+def test_fused_step_and_reencode_on_more_than_2_31_elements(big_weight, fmt):
+    """``adam_step_fp32_master`` on a quantised weight (one pass: step + payload) against
+    the plain step followed by ``copy_(master)``, whole tensors compared on the GPU."""
+    from offload_adam_amd import qweight
+    from offload_adam_amd.kernels import adam_step_fp32_master
+
+    cls = {"int8": qweight.Int8QWeight, "int4": qweight.Int4QWeight,
+           "nf4": qweight.NF4QWeight, "nvfp4": qweight.NVFP4QWeight}[fmt]
+    gen = torch.Generator(device="cuda").manual_seed(21)
+
+    def states():
+        st = {}
+        for name, std in (("grad", 1e-3), ("exp_avg", 1e-4), ("exp_avg_sq", 1e-3)):
+            t = torch.empty(ROWS * COLS, dtype=BF16, device="cuda")
+            fill_normal(t, std, gen)
+            st[name] = t.view(ROWS, COLS)
+        st["exp_avg_sq"].abs_()
+        st["master_params"] = big_weight.float()
+        return st
+
+    fused_w, plain_w = cls.from_float(big_weight), cls.from_float(big_weight)
+    fused_st = states()
+    plain_st = {k: v.clone() for k, v in fused_st.items()}
+    adam_step_fp32_master(fused_w, fused_st, *HYP, decoupled_weight_decay=True)
+    adam_step_fp32_master(None, plain_st, *HYP, decoupled_weight_decay=True)
+    plain_w.copy_(plain_st["master_params"])
+    torch.cuda.synchronize()
+
+    def same(a, b):
+        if a.dtype == torch.float8_e4m3fn:
+            a, b = a.view(torch.uint8), b.view(torch.uint8)
+        elif a.is_floating_point():
+            a = a.view(torch.int32 if a.element_size() == 4 else torch.int16)
+            b = b.view(a.dtype)
+        return torch.equal(a, b)
+
+    for k in ("exp_avg", "exp_avg_sq", "master_params"):
+        assert same(fused_st[k], plain_st[k]), k
+    for name in cls._PAYLOAD:
+        assert same(getattr(fused_w, name), getattr(plain_w, name)), name
+    # the payload moved, also past element 2^31
+    before = cls.from_float(big_weight[-8:].contiguous())
+    first = cls._PAYLOAD[0]
+    tail = getattr(cls.from_float(fused_st["master_params"][-8:].contiguous()), first)
+    assert not same(getattr(before, first), tail)
