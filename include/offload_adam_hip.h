@@ -18,7 +18,9 @@
  *   - return value: 0 on success, a positive hipError_t from the HIP runtime,
  *     or a negative OA_E* code for an argument the library rejects; nothing is
  *     launched when the return value is non-zero;
- *   - re-entrant, no global mutable state, never throws.
+ *   - re-entrant and never throws; no global mutable state, with one exception:
+ *     oa_grad_norm_bf16_static keeps its partial sums in a device array inside
+ *     the library (one per GPU) and caches that array's address per device.
  *
  * Element types: "bf16" = bfloat16 stored as uint16_t, "f32" = IEEE binary32,
  * "i16" = int16_t.  Scalars are binary32 because the reference's Triton
@@ -201,6 +203,28 @@ int oa_grad_norm_bf16(const void* grad, int64_t n, void* norm_out, void* sumsq_o
 #define OA_NORM_STATIC_MAX_ELEMS ((int64_t)1 << 31)  /* a 4 GiB bf16 gradient */
 int oa_grad_norm_bf16_static(const void* grad, int64_t n, void* norm_out,
                              void* sumsq_out, void* stream);
+
+/* Per-parameter norms of a whole list of gradients: what the loop of
+ * `torch.norm(grad, 2.0)` calls over the parameters amounts to on the last
+ * micro-batch (src/offload_adam/offload_adam.py:504-505, 531-532, read back by
+ * step() at :553-561), done with two launches per 36 gradients instead of one or
+ * two per gradient (tensor descriptors travel as kernel arguments).
+ *   count       number of gradients; every array below has `count` entries
+ *   grads       device pointers to bf16 gradients, any 2-byte alignment
+ *   numels      element counts (0 gives a norm of 0)
+ *   norm_outs   device pointers, ONE bf16 each (e.g. the slots of one buffer)
+ *   sumsq_outs  NULL, or device pointers to ONE f32 each (entries may be NULL)
+ *   workspace   device scratch for the partial sums, 64-byte aligned,
+ *               `workspace_bytes` long: at least oa_norm_workspace_bytes();
+ *               oa_norm_multi_workspace_bytes() lets every launch take its 36
+ *               gradients whatever their sizes.  Contents need no initialisation;
+ *               launches that may overlap need separate workspaces.
+ * Every argument is validated before the first launch.  Results are identical,
+ * bit for bit, to `count` calls of oa_grad_norm_bf16. */
+size_t oa_norm_multi_workspace_bytes(void);
+int oa_grad_norm_multi(int count, const void* const* grads, const int64_t* numels,
+                       void* const* norm_outs, void* const* sumsq_outs, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /* Replaces the global-norm and clip-coefficient arithmetic of
  * OffloadAdam.step (src/offload_adam/offload_adam.py:553-561):

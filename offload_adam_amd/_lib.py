@@ -58,6 +58,12 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
     ),
+    "oa_norm_multi_workspace_bytes": (c_size_t, []),
+    # count, grads, numels, norm_outs, sumsq_outs, workspace, workspace_bytes, stream
+    "oa_grad_norm_multi": (
+        c_int,
+        [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
     "oa_clip_coef_bf16": (
         c_int,
         [c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p],

@@ -361,8 +361,8 @@ adam_vec_kernel(const AdamArgs a, uint32_t tiles) {
 
 // Multi-tensor form: one launch covers up to kMultiMax parameters.  The
 // per-tensor pointers and scalars travel in the kernel arguments (no device
-// table, nothing to allocate); block b finds its tensor by scanning the
-// prefix sums of tiles, which is uniform per block.  Back-to-back tensors share
+// table, nothing to allocate); block b finds its tensor from the prefix sums of
+// tiles with one load and one ballot, the same value in every lane.  Back-to-back tensors share
 // one grid, so the ramp-up and drain of a launch are paid once per chunk
 // instead of once per parameter.
 constexpr int kMultiMax = 36;
@@ -387,8 +387,7 @@ __global__ void __launch_bounds__(Shape<MODE>::kThreads)
 adam_multi_kernel(const MultiArgs ma) {
   const uint32_t b = xcd_tile<Shape<MODE>::kChunk>(blockIdx.x);
   if (b >= ma.tile_start[ma.count]) return;
-  int t = 0;
-  while (t + 1 < ma.count && b >= ma.tile_start[t + 1]) ++t;
+  const int t = tensor_of_block(b, ma.tile_start, ma.count);
   AdamArgs a;
   a.p = ma.p[t];
   a.g = ma.g[t];

@@ -56,6 +56,13 @@ __device__ __forceinline__ float bf16hi_to_f32(uint32_t w) {
 // src/offload_adam/kernels/fp32_master.py:46-53 writes it: M is the fp32 value
 // being optimised, m / v the moments, omb = 1 - beta_hat.  One rounding per
 // operation; sqrt and divide are correctly rounded (compile flags).
+// Measurement switch, never set in the shipped build: 1 replaces the correctly
+// rounded square root and divide by the hardware's approximate v_sqrt_f32 and
+// v_rcp_f32 (about 20 instructions fewer per element).  Results then differ
+// from the reference's; it exists to show what the exact arithmetic costs.
+#ifndef OA_ADAM_APPROX_DIV_SQRT
+#define OA_ADAM_APPROX_DIV_SQRT 0
+#endif
 __device__ __forceinline__ void adam_core(float& M, float g, float& m, float& v, bool decoupled,
                                           float lr, float wd, float lr_wd, float omb1,
                                           float omb2, float eps) {
@@ -66,8 +73,13 @@ __device__ __forceinline__ void adam_core(float& M, float g, float& m, float& v,
   }
   m = m + omb1 * (g - m);
   v = v + omb2 * (g * g - v);
+#if OA_ADAM_APPROX_DIV_SQRT
+  const float denom = __builtin_amdgcn_sqrtf(v) + eps;
+  M = M - (lr * m) * __builtin_amdgcn_rcpf(denom);
+#else
   const float denom = sqrtf(v) + eps;
   M = M - (lr * m) / denom;
+#endif
 }
 
 // Philox4x32-10 (Salmon et al., SC'11): round multipliers 0xD2511F53 and
@@ -153,6 +165,18 @@ inline uint32_t xcd_grid(uint32_t tiles, uint32_t chunk) {
   return (tiles + q - 1) / q * q;
 }
 
+
+// Multi-tensor launches: `start[0..count]` are the prefix sums of the tensors'
+// workgroup counts (count < 64, every tensor has at least one workgroup) and b <
+// start[count].  Returns the tensor workgroup b belongs to, the same value in every
+// lane: lane j compares b with the end of tensor j and the wave counts the tensors
+// that end at or before b - one load and one ballot instead of a scan whose loads
+// depend on each other.
+__device__ __forceinline__ int tensor_of_block(uint32_t b, const uint32_t* start, int count) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const uint32_t end = lane < count ? start[lane + 1] : 0xFFFFFFFFu;
+  return __popcll(__ballot(b >= end));
+}
 
 inline bool aligned_to(const void* p, uintptr_t a) {
   return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;

@@ -70,19 +70,18 @@ __device__ __forceinline__ float sq8(const u32x4 w, float acc) {
   return acc;
 }
 
+// Sum of squares of one block's share of a gradient, the same value in every lane.
 // head = elements before the first 16-byte boundary, groups = aligned 8-element
-// groups after it; head and tail elements are folded in by block 0.  Block b
-// takes tiles b, b + gridDim.x, ... (one tile each unless the tensor has more
-// than kMaxBlocks tiles).
-__global__ void __launch_bounds__(kThreads)
-grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, int64_t groups,
-                         float* __restrict__ partial, uint16_t* __restrict__ norm_direct,
-                         float* __restrict__ sumsq_direct) {
-  __shared__ float lds[kThreads / kWave];
+// groups after it; head and tail elements are folded in by block 0.  Block b of
+// `blocks` takes tiles b, b + blocks, ... (one tile each unless the tensor has
+// more than kMaxBlocks tiles).
+__device__ __forceinline__ float block_sumsq(const uint16_t* __restrict__ g, int64_t n, int head,
+                                             int64_t groups, uint32_t block, uint32_t blocks,
+                                             float* lds) {
   const u32x4* body = reinterpret_cast<const u32x4*>(g + head);
   const int64_t tiles = (groups + kTileGroups - 1) / kTileGroups;
   float acc = 0.0f;
-  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+  for (int64_t tile = block; tile < tiles; tile += blocks) {
     const int64_t base = tile * kTileGroups + threadIdx.x;
     u32x4 w[kUnroll];
 #pragma unroll
@@ -94,7 +93,7 @@ grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, in
     for (int k = 0; k < kUnroll; ++k) acc = sq8(w[k], acc);
   }
 
-  if (blockIdx.x == 0) {
+  if (block == 0) {
     const int64_t tail_start = head + groups * 8;
     const int64_t extra = head + (n - tail_start);  // < 16
     if (threadIdx.x < extra) {
@@ -104,8 +103,15 @@ grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, in
       acc = fmaf(x, x, acc);
     }
   }
+  return block_sum<kThreads>(acc, lds);
+}
 
-  const float total = block_sum<kThreads>(acc, lds);
+__global__ void __launch_bounds__(kThreads)
+grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, int64_t groups,
+                         float* __restrict__ partial, uint16_t* __restrict__ norm_direct,
+                         float* __restrict__ sumsq_direct) {
+  __shared__ float lds[kThreads / kWave];
+  const float total = block_sumsq(g, n, head, groups, blockIdx.x, gridDim.x, lds);
   if (threadIdx.x == 0) {
     if (norm_direct) {
       // a one-block launch is its own final pass: the second launch would add this
@@ -118,10 +124,10 @@ grad_norm_partial_kernel(const uint16_t* __restrict__ g, int64_t n, int head, in
   }
 }
 
-__global__ void __launch_bounds__(kFinalThreads)
-grad_norm_final_kernel(const float* __restrict__ partial, int blocks,
-                       uint16_t* __restrict__ norm_out, float* __restrict__ sumsq_out) {
-  __shared__ float lds[kFinalThreads / kWave];
+// The fold of one tensor's partials, in index order, by one block of kFinalThreads lanes.
+__device__ __forceinline__ void fold_partials(const float* __restrict__ partial, int blocks,
+                                              uint16_t* __restrict__ norm_out,
+                                              float* __restrict__ sumsq_out, float* lds) {
   float s = 0.0f;
   for (int b = threadIdx.x; b < blocks; b += 4 * kFinalThreads) {
     float v[4];
@@ -137,6 +143,53 @@ grad_norm_final_kernel(const float* __restrict__ partial, int blocks,
     if (sumsq_out) *sumsq_out = s;
     *norm_out = (uint16_t)f32_to_bf16_1(sqrtf(s));
   }
+}
+
+__global__ void __launch_bounds__(kFinalThreads)
+grad_norm_final_kernel(const float* __restrict__ partial, int blocks,
+                       uint16_t* __restrict__ norm_out, float* __restrict__ sumsq_out) {
+  __shared__ float lds[kFinalThreads / kWave];
+  fold_partials(partial, blocks, norm_out, sumsq_out, lds);
+}
+
+// Multi-tensor form: one launch takes the partial sums of up to kNormMultiMax
+// gradients (descriptors travel as kernel arguments), a second one folds every
+// tensor's partials, one block per tensor.  Each tensor gets the block count, the
+// tile -> block map and the fold order of its own two-launch norm, so the results
+// are the same bits.  A gradient of a few thousand elements costs two launches
+// when it is taken alone; here a whole model's worth of them shares two.
+constexpr int kNormMultiMax = 36;
+
+struct NormMultiArgs {
+  const uint16_t* g[kNormMultiMax];
+  int64_t n[kNormMultiMax];
+  uint16_t* norm[kNormMultiMax];
+  float* sumsq[kNormMultiMax];
+  uint32_t block_start[kNormMultiMax + 1];  // first workgroup (= first partial) of each tensor
+  int count;
+};
+
+__global__ void __launch_bounds__(kThreads)
+grad_norm_multi_partial_kernel(const NormMultiArgs a, float* __restrict__ partial) {
+  __shared__ float lds[kThreads / kWave];
+  const uint32_t b = blockIdx.x;
+  const int t = tensor_of_block(b, a.block_start, a.count);
+  const uint16_t* g = a.g[t];
+  const int64_t n = a.n[t];
+  int64_t head = (int64_t)(((16 - (reinterpret_cast<uintptr_t>(g) & 15)) & 15) / 2);
+  if (head > n) head = n;
+  const int64_t groups = (n - head) / 8;
+  const float total = block_sumsq(g, n, (int)head, groups, b - a.block_start[t],
+                                  a.block_start[t + 1] - a.block_start[t], lds);
+  if (threadIdx.x == 0) partial[b] = total;
+}
+
+__global__ void __launch_bounds__(kFinalThreads)
+grad_norm_multi_final_kernel(const NormMultiArgs a, const float* __restrict__ partial) {
+  __shared__ float lds[kFinalThreads / kWave];
+  const int t = blockIdx.x;
+  fold_partials(partial + a.block_start[t], (int)(a.block_start[t + 1] - a.block_start[t]),
+                a.norm[t], a.sumsq[t], lds);
 }
 
 // total = bf16(sqrt(sum norms^2)); coef = min(bf16(bf16(1/bf16(total+1e-6)) * max_norm), 1)
@@ -173,9 +226,10 @@ extern "C" size_t oa_norm_workspace_bytes(void) { return sizeof(NormWorkspace); 
 namespace oa {
 namespace {
 
-// The two launches of a norm; `partial` holds at least kMaxBlocks floats.
-int launch_grad_norm(const void* grad, int64_t n, void* norm_out, void* sumsq_out,
-                     float* partial, hipStream_t s) {
+// Workgroups (= partials) of the first launch for a gradient at `grad`: one per
+// 32 KiB tile, at most kMaxBlocks; also yields the unaligned head and the number
+// of aligned 8-element groups.
+int64_t norm_blocks(const void* grad, int64_t n, int64_t* head_out, int64_t* groups_out) {
   const uintptr_t addr = reinterpret_cast<uintptr_t>(grad);
   int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / 2);
   if (head > n) head = n;
@@ -183,6 +237,16 @@ int launch_grad_norm(const void* grad, int64_t n, void* norm_out, void* sumsq_ou
   int64_t blocks = (groups + kTileGroups - 1) / kTileGroups;
   if (blocks < 1) blocks = 1;
   if (blocks > kMaxBlocks) blocks = kMaxBlocks;
+  if (head_out) *head_out = head;
+  if (groups_out) *groups_out = groups;
+  return blocks;
+}
+
+// The two launches of a norm; `partial` holds at least kMaxBlocks floats.
+int launch_grad_norm(const void* grad, int64_t n, void* norm_out, void* sumsq_out,
+                     float* partial, hipStream_t s) {
+  int64_t head = 0, groups = 0;
+  const int64_t blocks = norm_blocks(grad, n, &head, &groups);
   const bool single = blocks == 1;  // tensors of up to 16384 elements: one launch, not two
   hipLaunchKernelGGL(grad_norm_partial_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, s,
                      static_cast<const uint16_t*>(grad), n, (int)head, groups, partial,
@@ -251,6 +315,62 @@ extern "C" int oa_grad_norm_bf16_static(const void* grad, int64_t n, void* norm_
   // the array has to start at zero.
   return launch_grad_norm(grad, n, norm_out, sumsq_out, partial,
                           static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t oa_norm_multi_workspace_bytes(void) {
+  return sizeof(float) * (size_t)kNormMultiMax * kMaxBlocks;
+}
+
+extern "C" int oa_grad_norm_multi(int count, const void* const* grads, const int64_t* numels,
+                                  void* const* norm_outs, void* const* sumsq_outs,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  if (count < 0) return OA_EINVAL;
+  if (count == 0) return 0;
+  if (!grads || !numels || !norm_outs || !workspace) return OA_EINVAL;
+  if (workspace_bytes < sizeof(NormWorkspace)) return OA_EINVAL;  // one tensor must always fit
+  if (!aligned_to(workspace, 64)) return OA_EALIGN;
+  // Validate everything before the first launch.
+  for (int i = 0; i < count; ++i) {
+    if (numels[i] < 0 || !norm_outs[i] || (numels[i] > 0 && !grads[i])) return OA_EINVAL;
+    if (!aligned_to(grads[i], 2) || !aligned_to(norm_outs[i], 2) ||
+        (sumsq_outs && sumsq_outs[i] && !aligned_to(sumsq_outs[i], 4)))
+      return OA_EALIGN;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* partial = static_cast<float*>(workspace);
+  const uint64_t capacity = workspace_bytes / sizeof(float);  // partials one launch may write
+
+  NormMultiArgs a;
+  a.count = 0;
+  a.block_start[0] = 0;
+  auto flush = [&]() -> int {
+    if (a.count == 0) return 0;
+    hipLaunchKernelGGL(grad_norm_multi_partial_kernel, dim3(a.block_start[a.count]),
+                       dim3(kThreads), 0, s, a, partial);
+    int rc = launch_status();
+    if (rc) return rc;
+    hipLaunchKernelGGL(grad_norm_multi_final_kernel, dim3((unsigned)a.count),
+                       dim3(kFinalThreads), 0, s, a, partial);
+    a.count = 0;
+    return launch_status();
+  };
+  // Launches on one stream run in order: the next group's partials overwrite the
+  // workspace only after this group's fold has read it.
+  for (int i = 0; i < count; ++i) {
+    const uint64_t blocks = (uint64_t)norm_blocks(grads[i], numels[i], nullptr, nullptr);
+    if (a.count == kNormMultiMax || a.block_start[a.count] + blocks > capacity) {
+      int rc = flush();
+      if (rc) return rc;
+    }
+    const int j = a.count;
+    a.g[j] = static_cast<const uint16_t*>(grads[i]);
+    a.n[j] = numels[i];
+    a.norm[j] = static_cast<uint16_t*>(norm_outs[i]);
+    a.sumsq[j] = sumsq_outs ? static_cast<float*>(sumsq_outs[i]) : nullptr;
+    a.block_start[j + 1] = a.block_start[j] + (uint32_t)blocks;
+    a.count = j + 1;
+  }
+  return flush();
 }
 
 extern "C" int oa_clip_coef_bf16(const void* norms, int64_t count, float max_norm,

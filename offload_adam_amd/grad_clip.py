@@ -2,10 +2,11 @@
 
 Stand-ins for the torch calls of the reference's clipping path
 (src/offload_adam/offload_adam.py:504-505, 531-532, 553-561): one HIP launch
-per norm, one tiny launch for the coefficient, no host synchronisation.
+per norm (or two launches per 36 norms, ``grad_norms_``), one tiny launch for
+the coefficient, no host synchronisation.
 """
 
-from ctypes import c_float, c_int64
+from ctypes import c_float, c_int, c_int64, c_size_t, c_uint64
 
 import torch
 
@@ -48,6 +49,46 @@ def grad_norm_(grad, out):
         )
     _lib.check(code, "oa_grad_norm_bf16")
     return out
+
+
+_multi_workspaces = {}
+NORMS_PER_LAUNCH = 36  # gradients one pair of launches of ``grad_norms_`` takes
+
+
+def grad_norms_(grads, outs, validate=True):
+    """``grad_norm_(grads[i], outs[i])`` for every i, with two launches per 36
+    gradients instead of one or two per gradient.  Same bits as the single calls.
+
+    ``grads``: contiguous bf16 tensors on one GPU; ``outs``: one-element bf16
+    tensors on that GPU (typically 0-dim views of one buffer of slots)."""
+    count = len(grads)
+    if len(outs) != count:
+        raise ValueError("grads and outs must have the same length")
+    if count == 0:
+        return outs
+    dev = grads[0].device
+    for g, o in zip(grads, outs) if validate else ():
+        if g.dtype != torch.bfloat16 or o.dtype != torch.bfloat16:
+            raise TypeError("grad_norms_ works on bfloat16 tensors")
+        if not g.is_cuda or g.device != dev or o.device != dev:
+            raise ValueError("every gradient and output must be on the same GPU")
+        if not g.is_contiguous() or o.numel() != 1:
+            raise ValueError("gradients must be contiguous and outputs hold one element")
+    lib = _lib.load()
+    with _lib.device_guard(dev):
+        stream = _lib.current_stream_id()
+        key = (dev.index, stream)
+        ws = _multi_workspaces.get(key)
+        if ws is None:
+            ws = torch.empty(lib.oa_norm_multi_workspace_bytes(), dtype=torch.uint8, device=dev)
+            _multi_workspaces[key] = ws
+        g_tab = (c_uint64 * count)(*[g.data_ptr() for g in grads])
+        n_tab = (c_int64 * count)(*[g.numel() for g in grads])
+        o_tab = (c_uint64 * count)(*[o.data_ptr() for o in outs])
+        code = lib.oa_grad_norm_multi(c_int(count), g_tab, n_tab, o_tab, None, _lib.ptr(ws),
+                                      c_size_t(ws.numel()), _lib.c_void_p(stream))
+    _lib.check(code, "oa_grad_norm_multi")
+    return outs
 
 
 def grad_norm(grad):

@@ -60,6 +60,93 @@ def test_grad_norm_unaligned_and_reuse(oracle):
             assert _ulp_diff(got, oracle.grad_norm_bf16(bits(g))) <= 1, (off, n)
 
 
+def test_multi_tensor_norms_equal_single_calls(oracle):
+    """oa_grad_norm_multi: every slot holds the bits the per-gradient call writes
+    (same block counts, same fold order), for empty, tiny, ragged and unaligned
+    gradients, a gradient with more tiles than workgroups, and more gradients
+    than one launch takes; within one bf16 ulp of the oracle."""
+    from offload_adam_amd.grad_clip import grad_norm_, grad_norms_
+
+    gen = torch.Generator().manual_seed(11)
+    sizes = ([0, 1, 7, 8, 9, 4096, 4099, 16384, 16385, 65_536, (1 << 20) + 3]
+             + [4096] * 40 + [524_288] * 6 + [11_534_336, 3 * (1 << 28) // 2 + 5])
+    base = [(torch.randn(n + 8, generator=gen) * 5e-3).to(BF16).cuda() for n in sizes]
+    # every second gradient starts off a 16-byte boundary
+    grads = [b[(i % 2) * (1 + i % 7):][:n] for i, (b, n) in enumerate(zip(base, sizes))]
+    assert len(grads) > 36
+    single = torch.full((len(grads),), -1.0, dtype=BF16, device="cuda")
+    for i, g in enumerate(grads):
+        grad_norm_(g, single[i])
+    multi = torch.full((len(grads),), -1.0, dtype=BF16, device="cuda")
+    grad_norms_(grads, [multi[i] for i in range(len(grads))])
+    torch.cuda.synchronize()
+    assert bits(multi).tolist() == bits(single).tolist()
+    for i, g in enumerate(grads):
+        if g.numel() <= (1 << 24):
+            assert _ulp_diff(bits(multi[i:i + 1])[0], oracle.grad_norm_bf16(bits(g))) <= 1, i
+    # second call on the same workspace, fewer and smaller gradients
+    again = torch.full((5,), -1.0, dtype=BF16, device="cuda")
+    grad_norms_(grads[3:8], [again[i] for i in range(5)])
+    assert bits(again).tolist() == bits(single[3:8]).tolist()
+
+
+def test_multi_tensor_norm_c_abi_contract():
+    """Through the C ABI: a workspace of the single-tensor size still works (more
+    launches, same bits), sums of squares are optional per entry, bad arguments
+    are rejected before anything is written."""
+    import ctypes
+
+    from offload_adam_amd import _lib
+    from offload_adam_amd.grad_clip import grad_norm_
+
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(12)
+    sizes = [58_720_256, 16_777_216, 4096, 300_000_000, 1, 65_536]
+    grads = [(torch.randn(n, generator=gen) * 5e-3).to(BF16).cuda() for n in sizes]
+    count = len(grads)
+    want = torch.zeros(count, dtype=BF16, device="cuda")
+    for i, g in enumerate(grads):
+        grad_norm_(g, want[i])
+    small_ws = torch.empty(lib.oa_norm_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    assert lib.oa_norm_multi_workspace_bytes() == 36 * lib.oa_norm_workspace_bytes()
+    out = torch.full((count,), -1.0, dtype=BF16, device="cuda")
+    sumsq = torch.full((count,), -1.0, dtype=torch.float32, device="cuda")
+    g_tab = (ctypes.c_uint64 * count)(*[g.data_ptr() for g in grads])
+    n_tab = (ctypes.c_int64 * count)(*sizes)
+    o_tab = (ctypes.c_uint64 * count)(*[out[i].data_ptr() for i in range(count)])
+    s_tab = (ctypes.c_uint64 * count)(*[sumsq[i].data_ptr() if i % 2 == 0 else 0
+                                        for i in range(count)])
+    stream = _lib.current_stream_ptr()
+    rc = lib.oa_grad_norm_multi(count, g_tab, n_tab, o_tab, s_tab, small_ws.data_ptr(),
+                                small_ws.numel(), stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bits(out).tolist() == bits(want).tolist()
+    for i in range(count):
+        if i % 2 == 0:
+            assert bits(torch.sqrt(sumsq[i]).to(BF16).reshape(1))[0] == bits(out[i:i + 1])[0]
+        else:
+            assert sumsq[i].item() == -1.0
+    # rejected: workspace smaller than one tensor needs, negative size, null output
+    untouched = torch.full((count,), -1.0, dtype=BF16, device="cuda")
+    u_tab = (ctypes.c_uint64 * count)(*[untouched[i].data_ptr() for i in range(count)])
+    assert lib.oa_grad_norm_multi(count, g_tab, n_tab, u_tab, None, small_ws.data_ptr(),
+                                  small_ws.numel() - 64, stream) == -1
+    bad_n = (ctypes.c_int64 * count)(*([sizes[0], -1] + sizes[2:]))
+    assert lib.oa_grad_norm_multi(count, g_tab, bad_n, u_tab, None, small_ws.data_ptr(),
+                                  small_ws.numel(), stream) == -1
+    bad_o = (ctypes.c_uint64 * count)(*([untouched[0].data_ptr(), 0]
+                                        + [untouched[i].data_ptr() for i in range(2, count)]))
+    assert lib.oa_grad_norm_multi(count, g_tab, n_tab, bad_o, None, small_ws.data_ptr(),
+                                  small_ws.numel(), stream) == -1
+    odd = (ctypes.c_uint64 * count)(*([grads[0].data_ptr() + 1] + [g.data_ptr() for g in grads[1:]]))
+    assert lib.oa_grad_norm_multi(count, odd, n_tab, u_tab, None, small_ws.data_ptr(),
+                                  small_ws.numel(), stream) == -2
+    assert lib.oa_grad_norm_multi(0, None, None, None, None, None, 0, stream) == 0
+    torch.cuda.synchronize()
+    assert (untouched == -1.0).all()
+
+
 def test_clip_coef_matches_oracle_and_torch(oracle):
     from offload_adam_amd.grad_clip import clip_coef_
 
