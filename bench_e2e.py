@@ -204,12 +204,15 @@ def link_bytes_per_step(opt, grad_accum):
     # states and gradients kept on the GPU after their write-back are not fetched again
     states_in = state_b * sum(p.numel() for p in opt._offload_params
                               if p not in opt._state_cached)
-    if not opt.offload_grads:
+    # gradients that cross the link at all (not with offload_grads=False, nor those the
+    # pinned-memory limit keeps in HBM)
+    streamed = [p for p in opt._offload_params if p not in opt._grad_on_device]
+    if not streamed:
         return states_in, n * state_b
-    fetched = sum(p.numel() for p in opt._offload_params if p not in opt._grad_cached)
+    fetched = sum(p.numel() for p in streamed if p not in opt._grad_cached)
     # partial sums written to the host: all of them, or (write-back gradient cache)
     # only those that do not stay on the GPU
-    written = fetched if opt._grad_cache_write_back else n
+    written = fetched if opt._grad_cache_write_back else sum(p.numel() for p in streamed)
     passes = grad_accum - 1 if opt._step_in_backward else grad_accum
     h2d = states_in + fetched * 2 * passes
     d2h = n * state_b + written * 2 * passes
@@ -307,7 +310,23 @@ class StepCheck:
     its bf16 rounding.  Every sampled per-parameter norm must lie within one bf16
     ulp of the fp64 norm of the summed gradient, the total within one of the
     norm of all the slots, and the coefficient must equal the reference's bf16
-    expression ``clamp(max_norm / (total + 1e-6), max=1.0)`` bit for bit."""
+    expression ``clamp(max_norm / (total + 1e-6), max=1.0)`` bit for bit.
+
+    With ``fp32_master`` (the mode comparison of the reference's example, and every
+    ``--qat`` run) the moments are exact again, the fp32 master the optimizer left
+    behind must be the fp32 result of the update (same 1-ulp allowance), a plain
+    bf16 parameter must be the bf16 rounding of its master, and a quantised
+    parameter's payload must be, bit for bit, what the library's stand-alone encoder
+    (``copy_(master)`` into a clone) makes of that master, with its decoded value
+    within one quantisation step of the master."""
+
+    # decoded value against master, as a fraction of the largest magnitude of the
+    # element's row / group / block: the format's largest code error (int8 half of
+    # 1/127; int4 one step of 1/8, its largest value is clamped to code 7; NF4 half of
+    # the codebook's widest gap, 0.152; NVFP4 half of the 4..6 gap under an e4m3 scale
+    # that may be 1/16 off) plus 2^-8 each for a bf16 scale and the bf16 output
+    QAT_STEP_BOUND = {"Int8QWeight": 0.0125, "Int4QWeight": 0.134, "NF4QWeight": 0.157,
+                      "NVFP4QWeight": 0.19}
 
     def __init__(self, torch, model):
         self.torch, self.armed, self.grads, self.sample = torch, False, {}, {}
@@ -330,6 +349,8 @@ class StepCheck:
                     for p in self.sample}
         self.old_err = {p: opt.state[p]["rounding_error"].to(p.device, copy=True)
                         for p in self.sample if "rounding_error" in opt.state[p]}
+        self.old_master = {p: opt.state[p]["master_params"].to(p.device, copy=True)
+                           for p in self.sample if "master_params" in opt.state[p]}
         self.grads.clear()
         self.armed = True
 
@@ -375,6 +396,8 @@ class StepCheck:
         torch.cuda.synchronize()
         if opt.mode == "fp31_master":
             return self._after_fp31(opt)
+        if opt.mode == "fp32_master":
+            return self._after_fp32_master(opt)
         f32 = np.float32
         group = opt.param_groups[0]
         lr, eps, wd = float(f32(group["lr"])), float(f32(group["eps"])), group["weight_decay"]
@@ -424,9 +447,85 @@ class StepCheck:
         report["round_ups"] = int(ups)
         report["expected_round_ups"] = round(expected, 1)
         report["round_up_sigma"] = round(variance ** 0.5, 1)
-        report["unbiased_within_6_sigma"] = abs(ups - expected) < 6.0 * variance ** 0.5 + 1e3
+        # the fp32 result is known within one ulp per element, i.e. each round-up
+        # probability within 2^-16: that much systematic offset is allowed on top
+        report["unbiased_within_6_sigma"] = (abs(ups - expected)
+                                             < 6.0 * variance ** 0.5 + report["elements"] / 65536.0)
         report["passed"] = (report["moments_exact"] and report["params_on_bf16_neighbours"]
                             and report["unbiased_within_6_sigma"])
+        return report
+
+    def _after_fp32_master(self, opt):
+        import numpy as np
+
+        from offload_adam_amd.qweight.base import QWeightBase
+
+        torch = self.torch
+        f32 = np.float32
+        group = opt.param_groups[0]
+        lr, eps, wd = float(f32(group["lr"])), float(f32(group["eps"])), group["weight_decay"]
+        lr_wd = float(f32(group["lr"]) * f32(wd))
+        beta1, beta2 = group["betas"]
+        report = {"tensors": len(self.sample), "quantised_tensors": 0, "elements": 0,
+                  "moments_exact": True, "master_is_the_fp32_result": True,
+                  "param_is_bf16_of_the_master": True,
+                  "payload_is_the_encoding_of_the_master": True,
+                  "decoded_payload_within_one_step": True, "failed": []}
+        for p, name in self.sample.items():
+            step = opt.state[p]["step"]
+            b1h = (beta1**step - beta1) / (beta1**step - 1)
+            b2h = (beta2**step - beta2) / (beta2**step - 1)
+            omb1, omb2 = float(f32(1) - f32(b1h)), float(f32(1) - f32(b2h))
+            _, m0, v0 = self.old.pop(p)
+            m0, v0 = m0.float(), v0.float()
+            total = self.grads[p][0]
+            for g in self.grads[p][1:]:
+                total.add_(g)  # bf16 += bf16, as the optimizer accumulates
+            g = total.float()
+            m = m0 + omb1 * (g - m0)
+            v = v0 + omb2 * (g * g - v0)
+            m_now = opt.state[p]["exp_avg"].to(p.device)
+            v_now = opt.state[p]["exp_avg_sq"].to(p.device)
+            if not (torch.equal(m_now, m.to(torch.bfloat16))
+                    and torch.equal(v_now, v.to(torch.bfloat16))):
+                report["moments_exact"] = False
+                report["failed"].append(name + ": moments")
+            M0 = self.old_master.pop(p)
+            M = M0 - lr_wd * M0
+            M = M - (lr * m) / (torch.sqrt(v) + eps)
+            master = opt.state[p]["master_params"].to(p.device)
+            off = (master.view(torch.int32) - M.view(torch.int32)).abs() > 1
+            if bool((off & (master != M)).any()):
+                report["master_is_the_fp32_result"] = False
+                report["failed"].append(f"{name}: {int(off.sum())} masters off")
+            if isinstance(p.data, QWeightBase):
+                report["quantised_tensors"] += 1
+                q = p.data
+                again = q.detach().clone()
+                again.copy_(master)  # the stand-alone encoder on the master the step left
+                for key in q._PAYLOAD:
+                    a, b = getattr(q, key), getattr(again, key)
+                    if not torch.equal(a.reshape(-1).view(torch.uint8),
+                                       b.reshape(-1).view(torch.uint8)):
+                        report["payload_is_the_encoding_of_the_master"] = False
+                        report["failed"].append(f"{name}: payload {key}")
+                span = {"Int8QWeight": master.shape[1], "Int4QWeight": getattr(q, "group_size", 0),
+                        "NF4QWeight": getattr(q, "blocksize", 0), "NVFP4QWeight": 16}[type(q).__name__]
+                grouped = master.reshape(master.shape[0], -1, span)
+                err = (q.dequantize().float().reshape(grouped.shape) - grouped).abs()
+                bound = grouped.abs().amax(dim=-1, keepdim=True) * self.QAT_STEP_BOUND[type(q).__name__]
+                if bool((err > bound + 1e-30).any()):
+                    report["decoded_payload_within_one_step"] = False
+                    report["failed"].append(f"{name}: decoded payload off by more than a step")
+                del again, grouped, err, bound
+            elif not torch.equal(master.to(torch.bfloat16).view(torch.int16),
+                                 p.detach().view(torch.int16)):
+                report["param_is_bf16_of_the_master"] = False
+                report["failed"].append(name + ": param is not the bf16 rounding of its master")
+            report["elements"] += p.numel()
+            del m0, v0, g, m, v, M0, M, master, off
+        self.grads.clear()
+        report["passed"] = not report["failed"]
         return report
 
     def _after_fp31(self, opt):
@@ -536,11 +635,12 @@ def run(args):
 
     check = None
     if args.check:
-        if args.qat or not (
-                (args.mode == "stochastic_rounding" and args.max_grad_norm is None)
-                or args.mode == "fp31_master"):
-            raise SystemExit("--check covers the stochastic-rounding hook path (config 4) and "
-                             "fp31_master with or without clipping (config 2)")
+        if not ((args.mode == "stochastic_rounding" and args.max_grad_norm is None)
+                or args.mode == "fp31_master"
+                or (args.mode == "fp32_master" and args.max_grad_norm is None)):
+            raise SystemExit("--check covers the stochastic-rounding hook path (config 4), "
+                             "fp31_master with or without clipping (config 2) and the "
+                             "fp32_master hook path with plain or quantised (--qat) weights")
         check = StepCheck(torch, model)  # its hooks must precede the optimizer's
 
     compute_done = {}
@@ -598,6 +698,9 @@ def run(args):
     out["state_cache_GiB"] = round(
         sum(p.numel() for p in opt._state_cached) * (opt._bytes_per_elem_in_flight - 2) / 1024**3, 2)
     out["pinned_GiB"] = round(opt._estimate_pinned_bytes(opt._offload_params) / 1024**3, 2)
+    if opt.pinned_limit_report:
+        out["pinned_limit"] = {k: (round(v / 1024**3, 2) if k.endswith("_bytes") else v)
+                               for k, v in opt.pinned_limit_report.items()}
 
     timeline = None
     if args.copy_timeline:

@@ -22,6 +22,7 @@ What runs underneath is this package's HIP library: the fused AdamW kernels
 """
 
 import bisect
+import operator
 import sys
 import time
 import warnings
@@ -34,8 +35,8 @@ from . import _copy_engines, _lib, _trace, grad_clip
 from ._pretrained import stream_master_from_pretrained
 from .adam import _LOSSY_MASTER_HINT, MODE_TABLE
 from .kernels import adam_step_multi
-from .pinned_alloc import (alloc_pinned_states, numa_node_free_bytes, resolve_numa_target,
-                           zeros_pinned)
+from .pinned_alloc import (alloc_pinned_states, largest_grantable_bytes, numa_node_free_bytes,
+                           resolve_numa_target, zeros_pinned)
 from .qweight.base import QWeightBase
 
 _BF16 = torch.bfloat16
@@ -262,6 +263,18 @@ class OffloadAdam(Optimizer):
             ``prefetch_bytes`` left alone, that budget is added: states staged
             ahead of ``step()`` would hold the same HBM at the same time).
             Results are bit-identical.
+        pinned_limit_bytes (int | None, keyword-only): page-locked host memory the
+            optimizer may take.  ``None`` (default): what the GPU driver grants this
+            process (asked once at construction when more than 4 GiB are needed;
+            64 GiB per process on some systems, whatever the free RAM).  When the
+            states do not fit, the overflow stays in HBM instead of failing:
+            first the gradients of as many parameters as needed, in optimizer
+            order (for those, as with ``offload_grads=False``, the running sum
+            never leaves the GPU and ``state[p]`` holds no ``'grad'``), then
+            whole parameters (gradient and states resident, like the small ones
+            below ``inplace_param_threshold``).  One notice on stderr says what
+            was moved; ``RuntimeError`` only when HBM cannot take it either.
+            Results are bit-identical.
     """
 
     supported_modes = {
@@ -311,6 +324,7 @@ class OffloadAdam(Optimizer):
         state_cache_bytes=None,
         grad_cache_policy=None,
         spare_hbm=False,
+        pinned_limit_bytes=None,
     ):
         if prefetch_policy not in ("eager", "lazy"):
             raise ValueError(f"prefetch_policy must be 'eager' or 'lazy' (got {prefetch_policy!r})")
@@ -326,14 +340,27 @@ class OffloadAdam(Optimizer):
         self.offload_grads = bool(offload_grads)
         # Budgets: an int, 'auto' (a tenth of the HBM free at construction) or None,
         # which is the reference's contract unless spare_hbm asks for 'auto'.
-        for name, value in (("prefetch_bytes", prefetch_bytes),
-                            ("grad_cache_bytes", grad_cache_bytes),
-                            ("state_cache_bytes", state_cache_bytes)):
-            if value is None or value == "auto":
-                continue
-            if isinstance(value, bool) or not isinstance(value, int) or value < 0:
-                raise ValueError(f"{name} must be a non-negative int, 'auto' or None "
-                                 f"(got {value!r})")
+        def byte_count(name, value, auto_ok=True):
+            """An integer number of bytes: ints, numpy integers, floats such as 2e9."""
+            if value is None or (auto_ok and isinstance(value, str) and value == "auto"):
+                return value
+            ok = not isinstance(value, (bool, str))
+            if ok and isinstance(value, float):
+                ok = value.is_integer()
+            if ok:
+                try:
+                    value = int(value) if isinstance(value, float) else operator.index(value)
+                except TypeError:
+                    ok = False
+            if not ok or value < 0:
+                kinds = "a non-negative int, 'auto' or None" if auto_ok else "a non-negative int or None"
+                raise ValueError(f"{name} must be {kinds} (got {value!r})")
+            return value
+
+        prefetch_bytes = byte_count("prefetch_bytes", prefetch_bytes)
+        grad_cache_bytes = byte_count("grad_cache_bytes", grad_cache_bytes)
+        state_cache_bytes = byte_count("state_cache_bytes", state_cache_bytes)
+        self._pinned_limit_arg = byte_count("pinned_limit_bytes", pinned_limit_bytes, auto_ok=False)
         self.spare_hbm = bool(spare_hbm)
         if self.spare_hbm:
             prefetch_bytes = "auto" if prefetch_bytes is None else prefetch_bytes
@@ -351,10 +378,6 @@ class OffloadAdam(Optimizer):
             raise ValueError("grad_cache_policy must be 'write_back' or 'write_through' "
                              f"(got {grad_cache_policy!r})")
         self._grad_cache_write_back = grad_cache_policy == "write_back"
-        # what lives in pinned host memory between steps
-        self._host_config = {
-            k: d for k, d in self.offload_config.items() if k != "grad" or self.offload_grads
-        }
 
         self.max_grad_norm = max_grad_norm
         self._step_in_backward = max_grad_norm is None
@@ -399,6 +422,11 @@ class OffloadAdam(Optimizer):
             if p.numel() < inplace_param_threshold and p not in self._quant_params
         }
         self._offload_params = [p for p in params if p not in self._inplace_params]
+        # offloaded parameters whose running gradient sum never leaves the GPU: all of
+        # them with offload_grads=False, else those the pinned-memory limit displaces
+        self._grad_on_device = set() if self.offload_grads else set(self._offload_params)
+        self.pinned_limit_report = None  # what _fit_pinned_limit moved to HBM, if anything
+        self._fit_pinned_limit()
 
         def tenth_of_free_hbm():
             dev0 = self._offload_params[0].device
@@ -417,6 +445,8 @@ class OffloadAdam(Optimizer):
         if self.offload_grads and self._offload_params:
             budget = tenth_of_free_hbm() if grad_cache_bytes == "auto" else grad_cache_bytes
             for p in self._offload_params:
+                if p in self._grad_on_device:
+                    continue
                 nbytes = p.numel() * 2
                 if nbytes > budget:
                     break
@@ -545,9 +575,85 @@ class OffloadAdam(Optimizer):
                 self.device_states[p] = {}
                 state["host_grad_valid"] = False
 
+    def _host_keys(self, p):
+        """Names of the states of offloaded parameter ``p`` that live in pinned host memory."""
+        if p in self._grad_on_device:
+            return self._non_grad_keys
+        return self.offload_state_keys
+
     def _estimate_pinned_bytes(self, params):
-        per_elem = sum(torch.empty(0, dtype=d).element_size() for d in self._host_config.values())
-        return sum(p.numel() for p in params) * per_elem
+        size = {k: torch.empty(0, dtype=d).element_size() for k, d in self.offload_config.items()}
+        return sum(p.numel() * sum(size[k] for k in self._host_keys(p)) for p in params)
+
+    _PINNED_PROBE_FROM = 4 << 30   # requests below this are not pre-flighted
+    _PINNED_RESERVE = 1 << 30      # left to the rest of the process (loaders, staging probes)
+
+    def _fit_pinned_limit(self):
+        """Decide what stays in HBM when the pinned states exceed what the driver
+        grants (or ``pinned_limit_bytes``): gradients first, in optimizer order,
+        then whole parameters.  Runs before hooks, caches and buffers are set up."""
+        need = self._estimate_pinned_bytes(self._offload_params)
+        if not self._offload_params or self._offload_params[0].device.type != "cuda":
+            return
+        if self._pinned_limit_arg is not None:
+            budget = self._pinned_limit_arg
+        elif need < self._PINNED_PROBE_FROM:
+            return
+        else:
+            asked = need + self._PINNED_RESERVE
+            budget = largest_grantable_bytes(asked)
+            if budget >= asked:
+                return
+            budget -= self._PINNED_RESERVE
+        if need <= budget:
+            return
+        wanted = need
+        size = {k: torch.empty(0, dtype=d).element_size() for k, d in self.offload_config.items()}
+        state_b = sum(size[k] for k in self._non_grad_keys)
+        moved_grads = []
+        for p in self._offload_params:
+            if need <= budget:
+                break
+            if p not in self._grad_on_device:
+                self._grad_on_device.add(p)
+                moved_grads.append(p)
+                need -= p.numel() * size["grad"]
+        moved_whole = []
+        for p in self._offload_params:
+            if need <= budget:
+                break
+            if p in self._quant_params:
+                continue  # its fp32 master is re-encoded by the offloaded step only
+            moved_whole.append(p)
+            need -= p.numel() * state_b
+        if need > budget:
+            raise RuntimeError(
+                f"OffloadAdam: {wanted / _GIB:.1f} GiB of page-locked host memory are needed, "
+                f"{budget / _GIB:.1f} GiB may be taken, and what could move to HBM (every "
+                "gradient, every parameter that is not quantised) does not close the gap. "
+                "Page-locked memory is limited per process by the GPU driver, not by free RAM.")
+        whole = set(moved_whole)
+        hbm = (sum(p.numel() for p in moved_grads) * size["grad"]
+               + sum(p.numel() for p in moved_whole) * state_b)
+        free = torch.cuda.mem_get_info(self._offload_params[0].device)[0]
+        if hbm > free:
+            raise RuntimeError(
+                f"OffloadAdam: {wanted / _GIB:.1f} GiB of page-locked host memory are needed and "
+                f"{budget / _GIB:.1f} GiB may be taken; the remaining {hbm / _GIB:.1f} GiB do not "
+                f"fit the {free / _GIB:.1f} GiB of HBM that are free either.")
+        self._grad_on_device -= whole
+        self._inplace_params |= whole
+        self._offload_params = [p for p in self._offload_params if p not in whole]
+        self.pinned_limit_report = {
+            "needed_bytes": wanted, "limit_bytes": budget, "hbm_bytes": hbm,
+            "grads_in_hbm": len([p for p in moved_grads if p not in whole]),
+            "params_in_hbm": len(moved_whole),
+        }
+        print(f"OffloadAdam: {wanted / _GIB:.1f} GiB of page-locked host memory are needed, "
+              f"{budget / _GIB:.1f} GiB may be taken; kept in HBM instead ({hbm / _GIB:.1f} GiB): "
+              f"the gradients of {self.pinned_limit_report['grads_in_hbm']} parameters"
+              + (f" and all states of {len(moved_whole)} parameters" if moved_whole else ""),
+              file=sys.stderr)
 
     def _numa_precheck(self, params, numa_node):
         """Warn when the target NUMA node cannot hold the pinned budget: the soft
@@ -593,12 +699,13 @@ class OffloadAdam(Optimizer):
         # Every state of every parameter, carved out of a few large pinned arenas; the
         # arenas are all obtained (or the request refused as a whole) before any
         # value is written.
-        requests = [(p.shape, dtype) for p in params for dtype in self._host_config.values()]
+        requests = [(p.shape, self.offload_config[name]) for p in params
+                    for name in self._host_keys(p)]
         tensors = iter(alloc_pinned_states(requests, numa_node=numa_node))
         total = 0
         for p in params:
             state = self.state[p]
-            for name in self._host_config:
+            for name in self._host_keys(p):
                 t = next(tensors)
                 if name == "master_params":
                     t.copy_(p.data)  # widens bf16 losslessly; dequantises a quantised weight
@@ -644,7 +751,6 @@ class OffloadAdam(Optimizer):
         st = _copy_engines.status()
         if st["loaded"] or st["install"] == "off" or _copy_engine_warned:
             return
-        _copy_engine_warned = True
         why = {
             "late": "offload_adam_amd was imported after the GPU runtime had started",
             "missing": f"{_copy_engines.LIB_PATH.name} is not built "
@@ -652,12 +758,17 @@ class OffloadAdam(Optimizer):
             "unusable_path": f"the path of {_copy_engines.LIB_PATH.name} contains whitespace, "
                              "which HSA_TOOLS_LIB cannot name",
         }.get(st["install"], "the ROCr runtime did not load it from HSA_TOOLS_LIB")
-        warnings.warn(
+        message = (
             "OffloadAdam: host<->device copies are not pinned to fixed SDMA engines ("
             + why + "); expect a slower streaming step.  Import offload_adam_amd before "
-            "the first CUDA call, or set OFFLOAD_ADAM_COPY_ENGINES=off to silence this.",
-            stacklevel=3,
-        )
+            "the first CUDA call, start the script with `python -m offload_adam_amd.launch`, "
+            "or set OFFLOAD_ADAM_COPY_ENGINES=off to silence this.")
+        from . import _runtime_env
+
+        if _runtime_env.required():
+            raise RuntimeError("OFFLOAD_ADAM_REQUIRE_COPY_ENGINES is set: " + message)
+        _copy_engine_warned = True
+        warnings.warn(message, stacklevel=3)
 
     def _host_view(self, p, name):
         return self.state[p][name]
@@ -765,7 +876,7 @@ class OffloadAdam(Optimizer):
         """First micro-batch of a window adopts ``p.grad`` as the device gradient;
         later ones wait for the prefetched host gradient and add into it."""
         dev, state = self.device_states[p], self.state[p]
-        if not self.offload_grads:
+        if p in self._grad_on_device:
             # the running sum never leaves the GPU
             if dev.get("grad") is None:
                 dev["grad"] = p.grad
@@ -1040,11 +1151,10 @@ class OffloadAdam(Optimizer):
         if len(self._bw_prefix) != len(order) + 1:
             # bytes of device staging of order[:j], for the bisection below
             self._bw_prefix = [0]
-            grad_b = 2 if self.offload_grads else 0
             state_b = self._bytes_per_elem_in_flight - 2
             for q in order:
                 per_elem = ((0 if q in self._state_cached else state_b)
-                            + (0 if q in self._grad_cached else grad_b))
+                            + (0 if q in self._grad_cached or q in self._grad_on_device else 2))
                 self._bw_prefix.append(self._bw_prefix[-1] + q.numel() * per_elem)
         prefix = self._bw_prefix
         first = pos + 1
@@ -1096,7 +1206,7 @@ class OffloadAdam(Optimizer):
         count): the host->device direction is then busy for the whole pass
         and staged states would only queue ahead of the gradients backward waits
         for (measured: 2.86 s instead of 2.71 s per 8B step)."""
-        if self.offload_grads and any(
+        if any(
             self.state[p]["host_grad_valid"] and self.device_states[p].get("grad") is None
             for p in self._offload_params
         ):
@@ -1169,7 +1279,7 @@ class OffloadAdam(Optimizer):
                 # offload_grads=False): stage the states the next step touches
                 # first now, up to the prefetch budget.
                 self._prefetch_ahead(-1, states_too=True)
-        elif self.offload_grads:
+        elif p not in self._grad_on_device:
             if p not in self._grad_cached:
                 self._issue_d2h(p, ["grad"])
             elif self._grad_cache_write_back:

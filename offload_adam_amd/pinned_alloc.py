@@ -10,13 +10,21 @@ threads, and released when the last tensor that views it is collected.
 
 ``PinnedArena`` / ``alloc_pinned_states`` are this package's own: the optimizer
 states of a model are carved out of a few large allocations (on 4 KiB
-boundaries) instead of one runtime allocation per state, after a pre-flight
-that fails before any memory is touched when the runtime will not grant the
-total.
+boundaries) instead of one runtime allocation per state.  The arenas are
+obtained one after another (each zero-filled as it arrives) before any caller
+data moves; when the runtime refuses one, those already held are released and
+the error names what the runtime would still grant.  ``OffloadAdam`` asks
+``largest_grantable_bytes`` first and keeps what does not fit in HBM.
+
+A state carved from an arena is a view of that arena's storage: ``torch.save``
+of such a tensor writes the whole arena (up to 8 GiB), and the arena's memory is
+returned only when every tensor carved from it is gone.  ``detached`` gives
+copies that own their storage, for saving a subset of the states.
 """
 
 import ctypes
 import os
+import time
 import weakref
 from pathlib import Path
 
@@ -179,15 +187,42 @@ class PinnedArena:
         return piece.view(dtype).view(shape)
 
 
+def detached(states):
+    """Copies of pinned states that own their storage (plain CPU tensors).
+
+    ``states``: a tensor, or a dict / list / tuple of them, nested as in
+    ``optimizer.state_dict()``; anything that is not a tensor is passed through.
+    Use it before ``torch.save`` of a subset of an ``OffloadAdam``'s states: the
+    optimizer's own tensors are views into shared arenas, and serialising a view
+    writes the whole arena behind it."""
+    if isinstance(states, torch.Tensor):
+        return states.detach().clone()
+    if isinstance(states, dict):
+        return {k: detached(v) for k, v in states.items()}
+    if isinstance(states, (list, tuple)):
+        return type(states)(detached(v) for v in states)
+    return states
+
+
 def largest_grantable_bytes(upper):
     """Largest single page-locked allocation the runtime grants right now, up to
-    ``upper`` bytes, to 256 MiB (bisection over allocate-and-release probes that
-    touch no page)."""
+    ``upper`` bytes, to 256 MiB (allocate-and-release probes that touch no page).
+
+    A refusal by the driver's per-process limit returns at once, while a probe that
+    succeeds costs about 40 ms per GiB, so the search walks down from ``upper`` while
+    probes are refused and stops at the first success; should refusals turn slow (a
+    host that is really out of memory) it falls back to bisection."""
     lib = _lib.load()
     step = 256 << 20
-    lo, hi = 0, max(1, -(-upper // step))
+    hi = max(1, -(-upper // step))
     if lib.oa_pinned_probe(ctypes.c_size_t(hi * step)) == 0:
         return hi * step
+    deadline = time.monotonic() + 2.0
+    while hi > 1 and time.monotonic() < deadline:
+        hi -= 1
+        if lib.oa_pinned_probe(ctypes.c_size_t(hi * step)) == 0:
+            return hi * step
+    lo = 0
     while hi - lo > 1:
         mid = (lo + hi) // 2
         if lib.oa_pinned_probe(ctypes.c_size_t(mid * step)) == 0:

@@ -152,6 +152,70 @@ def test_copies_run_on_the_fixed_engines_and_move_the_right_bytes():
     assert st2["h2d_copies"] == st1["h2d_copies"]
 
 
+_LATE = (
+    "import sys, warnings, torch\n"
+    "torch.zeros(1, device='cuda')  # the GPU runtime starts before the package is imported\n"
+    "import offload_adam_amd\n"
+    "from offload_adam_amd import OffloadAdam, _copy_engines, _runtime_env\n"
+    "model = torch.nn.Sequential(torch.nn.Linear(64, 64, bias=False)).to(device='cuda', dtype=torch.bfloat16)\n"
+    "with warnings.catch_warnings(record=True) as caught:\n"
+    "    warnings.simplefilter('always')\n"
+    "    OffloadAdam(model, inplace_param_threshold=0)\n"
+    "st = _copy_engines.status()\n"
+    "late = [w for w in caught if 'not pinned to fixed SDMA engines' in str(w.message)]\n"
+    "print(st['install'], st['loaded'], st['active'], len(late),\n"
+    "      'offload_adam_amd.launch' in str(late[0].message) if late else None,\n"
+    "      _runtime_env.prepare()['copy_engines'])"
+)
+
+
+@pytest.mark.gpu
+def test_an_import_after_the_first_gpu_call_warns_and_reports_late():
+    """The trap a reference user walks into with ``model.cuda()`` above the import:
+    the environment edit comes too late, the optimizer says so once, and ``status()``
+    shows why; with OFFLOAD_ADAM_REQUIRE_COPY_ENGINES the import raises instead."""
+    assert _run(_LATE) == "late False False 1 True late"
+    full = dict(os.environ, OFFLOAD_ADAM_REQUIRE_COPY_ENGINES="1")
+    full.pop("HSA_TOOLS_LIB", None)
+    res = subprocess.run([sys.executable, "-c", _LATE], capture_output=True, text=True, env=full,
+                         cwd=str(ROOT), timeout=300)
+    assert res.returncode != 0
+    assert "OFFLOAD_ADAM_REQUIRE_COPY_ENGINES is set" in res.stderr
+    assert "python -m offload_adam_amd.launch" in res.stderr
+
+
+@pytest.mark.gpu
+def test_the_launcher_takes_the_import_order_out_of_the_script(tmp_path):
+    """The same script started through ``python -m offload_adam_amd.launch``: the
+    library is in effect although the script touches the GPU before its import."""
+    script = tmp_path / "late_import.py"
+    script.write_text(_LATE.replace("print(st['install']", "print(sys.argv[1:], st['install']"))
+    full = dict(os.environ)
+    full.pop("HSA_TOOLS_LIB", None)
+    res = subprocess.run([sys.executable, "-m", "offload_adam_amd.launch", str(script), "--flag", "7"],
+                         capture_output=True, text=True, env=full, cwd=str(ROOT), timeout=300)
+    assert res.returncode == 0, res.stderr
+    assert res.stdout.strip().splitlines()[-1] == "['--flag', '7'] installed True True 0 None installed"
+
+
+def test_the_launcher_prints_the_environment_for_a_shell():
+    from offload_adam_amd import _copy_engines
+
+    full = dict(os.environ, HSA_TOOLS_LIB="/some/other/tool.so")
+    full.pop("GPU_MAX_HW_QUEUES", None)
+    res = subprocess.run([sys.executable, "-m", "offload_adam_amd.launch", "--print-env"],
+                         capture_output=True, text=True, env=full, cwd=str(ROOT), timeout=300)
+    assert res.returncode == 0, res.stderr
+    lines = res.stdout.strip().splitlines()
+    assert lines == [f"export HSA_TOOLS_LIB='{_copy_engines.LIB_PATH} /some/other/tool.so'",
+                     "export GPU_MAX_HW_QUEUES='8'"]
+    # a value the user exported stands
+    res = subprocess.run([sys.executable, "-m", "offload_adam_amd.launch", "--print-env"],
+                         capture_output=True, text=True, env=dict(full, GPU_MAX_HW_QUEUES="6"),
+                         cwd=str(ROOT), timeout=300)
+    assert res.stdout.strip().splitlines()[-1] == "export GPU_MAX_HW_QUEUES='6'"
+
+
 def test_roctx_ranges_are_off_by_default_and_load_on_request():
     from offload_adam_amd import _trace
 

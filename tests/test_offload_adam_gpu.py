@@ -1420,3 +1420,127 @@ def test_clipping_path_gives_its_spare_staging_budget_to_the_state_cache():
     assert sized._prestage_bytes == sized._PREFETCH_BYTES and not sized._state_cached
     plain = build(max_grad_norm=1.0)
     assert plain._prestage_bytes == plain._PREFETCH_BYTES and not plain._state_cached
+
+
+# ----------------------------------------------- pinned memory beyond the limit
+
+
+def _pinned_need(mode, **kw):
+    model, opt = run_offload_adam(mode, steps=0, ga=1, **kw)
+    return opt._estimate_pinned_bytes(opt._offload_params), opt
+
+
+@pytest.mark.parametrize("mode,kw", [
+    ("stochastic_rounding", dict()),
+    ("fp32_master", dict()),
+    ("fp31_master", dict(max_grad_norm=0.05)),
+])
+@pytest.mark.parametrize("ga", [1, 3])
+@pytest.mark.parametrize("fraction", [0.9, 0.55])
+def test_states_beyond_the_pinned_limit_stay_in_hbm(fixed_seed, capsys, mode, kw, ga, fraction):
+    """A limit below what the states need is a placement decision, not an error:
+    gradients stay in HBM first (0.9 of the need), then whole parameters (0.55: less
+    than the states without any gradient); one notice; results bit-identical to the
+    unconstrained run; the host never holds more than the limit."""
+    need, free_opt = _pinned_need(mode, **kw)
+    assert free_opt.pinned_limit_report is None and not free_opt._grad_on_device
+    n_offloaded = len(free_opt._offload_params)
+    ref_model, ref_opt = run_offload_adam(mode, steps=3, ga=ga, decoupled_weight_decay=True, **kw)
+    capsys.readouterr()
+    limit = int(need * fraction)
+    model, opt = run_offload_adam(mode, steps=3, ga=ga, decoupled_weight_decay=True,
+                                  pinned_limit_bytes=limit, **kw)
+    err = capsys.readouterr().err
+    assert err.count("page-locked host memory are needed") == 1 and "kept in HBM instead" in err
+    report = opt.pinned_limit_report
+    assert report["needed_bytes"] == need and report["limit_bytes"] == limit
+    assert opt._estimate_pinned_bytes(opt._offload_params) <= limit
+    pinned = sum(t.numel() * t.element_size() for p in opt._offload_params
+                 for t in opt.state[p].values() if torch.is_tensor(t) and t.is_pinned())
+    assert pinned == opt._estimate_pinned_bytes(opt._offload_params)
+    assert report["grads_in_hbm"] + report["params_in_hbm"] > 0
+    if fraction < 0.6:
+        assert report["params_in_hbm"] > 0 and len(opt._offload_params) < n_offloaded
+        assert all(p in opt._grad_on_device for p in opt._offload_params)
+    else:
+        assert report["params_in_hbm"] == 0 and 0 < len(opt._grad_on_device) < n_offloaded
+    assert_same_params(ref_model, model)
+    for pr, p in zip(ref_model.parameters(), model.parameters()):
+        for key in opt._non_grad_keys:
+            a, b = ref_opt.state[pr][key], opt.state[p][key]
+            assert torch.equal(a.cpu().view(torch.uint8), b.cpu().view(torch.uint8)), key
+        if p in opt._grad_on_device:
+            assert "grad" not in opt.state[p]
+
+
+def test_quantised_weights_keep_their_masters_on_the_host_under_a_limit(capsys):
+    """Quantised parameters are never made resident; when nothing else can move,
+    the constructor raises and says why."""
+    from offload_adam_amd import OffloadAdam
+    from offload_adam_amd.qweight import Int8QWeight, quantize_linears
+
+    def build(limit):
+        model = make_model(0)
+        quantize_linears(model, Int8QWeight)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            return OffloadAdam(model, mode="fp32_master", inplace_param_threshold=0,
+                               pinned_limit_bytes=limit)
+
+    free = build(None)
+    need = free._estimate_pinned_bytes(free._offload_params)
+    quant_states = sum(p.numel() for p in free._quant_params) * 8
+    opt = build(quant_states + 4096)
+    offloaded = {id(p) for p in opt._offload_params}  # (== is not defined for quantised weights)
+    assert all(id(p) in offloaded for p in opt._quant_params)
+    assert opt.pinned_limit_report["params_in_hbm"] > 0
+    with pytest.raises(RuntimeError, match="does not close the gap"):
+        build(quant_states - 4096)
+    assert need > quant_states
+
+
+@pytest.mark.parametrize("value,ok", [(2 ** 20, True), (2e6, True), (2.5, False), (-1, False),
+                                      ("auto", False), (True, False)])
+def test_byte_budgets_accept_any_integral_number(value, ok):
+    """numpy integers and integral floats are byte counts too; 'auto' only where it means something."""
+    import numpy as np
+
+    from offload_adam_amd import OffloadAdam
+
+    def build(**kw):
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            return OffloadAdam(make_model(0), inplace_param_threshold=5000, **kw)
+
+    if ok:
+        assert build(pinned_limit_bytes=value)._pinned_limit_arg == int(value)
+        assert build(prefetch_bytes=np.int64(value))._PREFETCH_BYTES == int(value)
+        assert build(grad_cache_bytes=value, state_cache_bytes=np.int32(4096)) is not None
+    else:
+        with pytest.raises(ValueError, match="pinned_limit_bytes"):
+            build(pinned_limit_bytes=value)
+        if value != "auto":
+            with pytest.raises(ValueError, match="prefetch_bytes"):
+                build(prefetch_bytes=value)
+
+
+def test_saving_one_carved_state_writes_its_arena_and_detached_does_not(tmp_path):
+    """States carved from one arena share its storage: ``torch.save`` of one of them
+    serialises the arena; ``pinned_alloc.detached`` gives copies that stand alone."""
+    from offload_adam_amd.pinned_alloc import alloc_pinned_states, detached
+
+    a, b, c = alloc_pinned_states([((1000,), torch.float32), ((300_000,), BF16),
+                                   ((70_000,), torch.int16)], numa_node=None)
+    a.fill_(1.5)
+    arena_bytes = a.untyped_storage().nbytes()
+    assert arena_bytes >= 4096 + 600_064 + 140_000
+    assert b.untyped_storage().data_ptr() == a.untyped_storage().data_ptr()
+    torch.save(a, tmp_path / "view.pt")
+    assert (tmp_path / "view.pt").stat().st_size >= arena_bytes
+    own = detached({"state": {0: {"exp_avg": a, "step": 3}}, "list": [c]})
+    assert own["state"][0]["step"] == 3 and torch.equal(own["state"][0]["exp_avg"], a)
+    assert own["state"][0]["exp_avg"].untyped_storage().nbytes() == 4000
+    torch.save(own["state"][0]["exp_avg"], tmp_path / "own.pt")
+    assert (tmp_path / "own.pt").stat().st_size < 4000 + 4096
+    loaded = torch.load(tmp_path / "own.pt", weights_only=True)
+    assert torch.equal(loaded, a)
