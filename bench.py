@@ -22,7 +22,11 @@ After the timed region of the default workload the same line also carries
   HBM caches, the same model with the GPU-resident ``Adam``, and config 2 as a
   training step (fp31_master with the clipping path);
 * ``offloaded_step_1b``: config 1 as a training step (the 1.1B set streamed, one
-  micro-batch per step).
+  micro-batch per step);
+* ``mode_comparison_8b`` and ``qat_step``: the reference's rounding-mode and QAT
+  tables as training steps through ``OffloadAdam``, each with a numerical check;
+* ``summary`` (the LAST key): roofline fraction per config and, per streamed step,
+  time, exposed optimizer time, link use, peak HBM and the check's verdict.
 
 ``--only-main`` stops after the timed region.  Only one GPU is used;
 ``--gpus N`` with N > 1 exits with a message.
@@ -381,20 +385,30 @@ def time_adam_workload(name, steps, warmup, *, rng=None, per_tensor=False, use_e
 
 
 def config0_row(steps=400, warmup=20):
-    """Benchmark config 0 on the GPU: the same 335 MB of operands every step (what
-    the config describes), and rotating through six operand sets so that the
-    256 MiB memory-side cache cannot serve any of it."""
+    """Benchmark config 0 on the GPU.  The row's ``roofline`` is the HBM figure:
+    six operand sets in rotation, so that the 256 MiB memory-side cache cannot serve
+    any of the 335 MB a step touches.  ``cache_assisted`` is the same kernel on the
+    same operands every step (what the config literally describes), part of which
+    that cache serves: not an HBM bandwidth."""
     import torch
 
-    row = {}
+    row = {"workload": "fp32_master, one flat tensor of 16,777,216 elements, 20 B/elem",
+           "floor_us_at_8TBps": 41.94}
+    # (the short same-operand run goes first: right after gigabytes of HBM are handed
+    # back, the driver's clearing of the freed pages competes with a 20 ms measurement)
     for label, sets in (("same_operands", 1), ("rotating_6_sets", 6)):
         r = time_adam_workload("c0_fp32_master_16m", steps, warmup, sets=sets)
-        row[label] = {"ms_per_step": round(r["elapsed_s"] / steps * 1e3, 4),
-                      "GBps_wall": round(r["bytes_per_step"] * steps / r["elapsed_s"] / 1e9, 1),
-                      "roofline": r["roofline"]}
+        entry = {"ms_per_step": round(r["elapsed_s"] / steps * 1e3, 4),
+                 "GBps_wall": round(r["bytes_per_step"] * steps / r["elapsed_s"] / 1e9, 1),
+                 "roofline": r["roofline"]}
+        if sets > 1:
+            row["roofline"] = r["roofline"]
+            row["hbm_cold"] = entry
+        else:
+            entry["note"] = ("335 MB of operands reused every step; the 256 MiB memory-side "
+                             "cache serves part of them")
+            row["cache_assisted"] = entry
         torch.cuda.empty_cache()
-    row["workload"] = "fp32_master, one flat tensor of 16,777,216 elements, 20 B/elem"
-    row["floor_us_at_8TBps"] = 41.94
     return row
 
 
@@ -524,6 +538,7 @@ def other_configs(cpu=True):
     out = {}
     for name, fn in (("c0_fp32_master_16m", config0_row), ("c2_fp31_clip_llama8b", config2_row),
                      ("c3_codecs", config3_row)):
+        progress(f"other config {name}")
         try:
             out[name] = fn()
         except Exception as exc:  # a failed side measurement must not lose the main line
@@ -538,9 +553,19 @@ def other_configs(cpu=True):
     return out
 
 
+_T0 = time.time()
+
+
+def progress(what):
+    """One line on stderr per finished section: a run of several minutes must not
+    look hung to whoever watches its output (stdout carries the JSON line only)."""
+    print(f"[bench.py +{time.time() - _T0:5.0f} s] {what}", file=sys.stderr, flush=True)
+
+
 def run_e2e(extra, steps, warmup, timeout_s, model="llama8b"):
     import subprocess
 
+    progress(f"bench_e2e.py --model {model} {' '.join(extra)}")
     cmd = [sys.executable, str(ROOT / "bench_e2e.py"), "--model", model, "--steps", str(steps),
            "--warmup", str(warmup)] + extra
     try:
@@ -558,7 +583,7 @@ def run_e2e(extra, steps, warmup, timeout_s, model="llama8b"):
             "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak", "link_floor_s", "pinned_GiB",
             "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB",
             "peak_gpu_GiB", "optimizer_init_s", "copy_engines", "transfer_streams", "check",
-            "max_grad_norm",
+            "max_grad_norm", "qat", "model_gpu_GiB", "pinned_limit",
             "loss_finite")
     row = {k: full[k] for k in keep if k in full}
     peak = (full.get("link_peak") or {}).get("bidir_each_GBps")
@@ -586,12 +611,100 @@ def offloaded_step_8b():
     return {
         "model": "llama8b (32 layers, hidden 4096, vocab 128256), bf16, 1 x 4096 tokens x 4 "
                  "micro-batches, activation checkpointing",
-        "reference_traffic": run_e2e(["--check"], steps=5, warmup=2, timeout_s=300),
-        "spare_hbm": run_e2e(["--spare-hbm"], steps=8, warmup=2, timeout_s=300),
-        "resident_adam": run_e2e(["--optimizer", "adam"], steps=4, warmup=1, timeout_s=300),
+        "reference_traffic": run_e2e(["--check"], steps=4, warmup=2, timeout_s=300),
+        "spare_hbm": run_e2e(["--spare-hbm"], steps=4, warmup=2, timeout_s=300),
+        "resident_adam": run_e2e(["--optimizer", "adam"], steps=3, warmup=1, timeout_s=300),
         "clip_path_fp31": run_e2e(["--mode", "fp31_master", "--max-grad-norm", "1.0", "--check"],
                                   steps=3, warmup=1, timeout_s=300),
     }
+
+
+def mode_comparison_8b():
+    """The reference's rounding-mode table (examples/e2e_train/README.md:99-109: one
+    micro-batch of 4096 tokens per step, offloading on) on the same 8B-shaped model,
+    both rows with ``OffloadAdam`` as constructed by default.  ``fp32_master`` needs
+    74.8 GiB of pinned host memory at this size; where the driver grants less, the
+    optimizer keeps the overflow (gradients first) in HBM and says so in
+    ``pinned_limit``."""
+    common = ["--grad-accum", "1"]
+    return {
+        "stochastic_rounding": run_e2e(common, steps=4, warmup=2, timeout_s=300),
+        "fp32_master": run_e2e(common + ["--mode", "fp32_master", "--check"], steps=3, warmup=1,
+                               timeout_s=300),
+    }
+
+
+def qat_steps():
+    """The reference's QAT table (examples/qat/README.md:121-130: ``fp32_master``,
+    one micro-batch of 8192 tokens per step, every attention / MLP projection
+    quantised, lm_head in bf16) through ``OffloadAdam`` as constructed by default,
+    each followed by the numerical check of one more step: the four formats and the
+    unquantised row on the 1.1B-shaped model, and int4 (the example's own command)
+    on the 8B-shaped one."""
+    common = ["--grad-accum", "1", "--seq", "8192", "--check"]
+    rows = {"llama1b": {"none": run_e2e(common + ["--mode", "fp32_master"], steps=5, warmup=2,
+                                        timeout_s=200, model="llama1b")}}
+    for fmt in ("int8", "int4", "nf4", "nvfp4"):
+        rows["llama1b"][fmt] = run_e2e(common + ["--qat", fmt], steps=5, warmup=2, timeout_s=200,
+                                       model="llama1b")
+    rows["llama8b"] = {"int4": run_e2e(common + ["--qat", "int4"], steps=3, warmup=1,
+                                       timeout_s=300)}
+    return rows
+
+
+def _step_summary(row):
+    """One streamed-step row boiled down for the summary at the end of the line."""
+    if not isinstance(row, dict) or "step_s" not in row:
+        return {"error": (row or {}).get("error", "missing")[:60]} if isinstance(row, dict) else None
+    out = {"s": row["step_s"], "exposed": row.get("exposed_optimizer_s"),
+           "GiB": row.get("peak_gpu_GiB")}
+    if "h2d_frac_of_bidir_peak" in row:
+        out["h2d"], out["d2h"] = row["h2d_frac_of_bidir_peak"], row["d2h_frac_of_bidir_peak"]
+    if "check" in row:
+        out["ok"] = bool(row["check"].get("passed"))
+    return out
+
+
+def summary_of(out):
+    """The figures a reader wants first, small enough to survive a log that keeps
+    only the end of the line: roofline fraction per config, and per streamed step
+    its time, exposed optimizer time, link use against the bidirectional peak, peak
+    HBM and whether its numerical check passed."""
+    def frac(d):
+        return (d or {}).get("frac") if isinstance(d, dict) else None
+
+    other = out.get("other_configs", {})
+    c0, c2, c3 = (other.get(k, {}) for k in ("c0_fp32_master_16m", "c2_fp31_clip_llama8b",
+                                             "c3_codecs"))
+    kernels = c3.get("kernels", []) if isinstance(c3, dict) else []
+
+    def least(pred):
+        vals = [k["frac"] for k in kernels if pred(k["kernel"]) and "frac" in k]
+        return min(vals) if vals else None
+
+    fr = {"c1": frac(out.get("roofline")),
+          "c1_ref_bits": frac(out.get("roofline_reference_layout")),
+          "c0_cold": frac(c0.get("roofline")),
+          "c0_cached": frac((c0.get("cache_assisted") or {}).get("roofline")),
+          "c2_step": frac((c2.get("adam_leg") or {}).get("roofline")),
+          "c2_norm": frac((c2.get("norm_leg") or {}).get("roofline")),
+          "c3_enc_min": least(lambda k: k.startswith("quant_") or k.startswith("nvfp4_amax")),
+          "c3_dec_min": least(lambda k: k.startswith("dequant_")),
+          "c3_fused_min": least(lambda k: k.endswith(", fused"))}
+    steps = {}
+    e8 = out.get("offloaded_step_8b", {})
+    for key, name in (("reference_traffic", "8b_ref"), ("spare_hbm", "8b_spare"),
+                      ("resident_adam", "8b_adam"), ("clip_path_fp31", "8b_clip")):
+        if key in e8:
+            steps[name] = _step_summary(e8[key])
+    if "offloaded_step_1b" in out:
+        steps["1b"] = _step_summary(out["offloaded_step_1b"])
+    for key, row in out.get("mode_comparison_8b", {}).items():
+        steps["8b_ga1_" + ("sr" if key == "stochastic_rounding" else "fp32m")] = _step_summary(row)
+    for model, rows in out.get("qat_step", {}).items():
+        for fmt, row in rows.items():
+            steps[f"qat_{model[5:]}_{fmt}"] = _step_summary(row)
+    return {"frac": fr, "steps": steps}
 
 
 def main():
@@ -614,8 +727,8 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip configs 0, 2 and 3 (about half a minute)")
     ap.add_argument("--no-e2e", action="store_true",
-                    help="skip the 8B training steps (bench_e2e.py, four child processes after "
-                         "the timed region; two to three minutes)")
+                    help="skip the training steps (bench_e2e.py in child processes after the timed "
+                         "region; about four minutes)")
     ap.add_argument("--no-events", action="store_true",
                     help="skip per-launch HIP events (used for profiler runs)")
     args = ap.parse_args()
@@ -648,7 +761,6 @@ def main():
 
     r = time_adam_workload(args.workload, args.steps, args.warmup, rng=args.rng,
                            per_tensor=args.per_tensor, use_events=not args.no_events)
-    torch.cuda.empty_cache()
     ms_per_step = r["elapsed_s"] / args.steps * 1e3
     value = r["bytes_per_step"] * args.steps / r["elapsed_s"] / 1e9
 
@@ -679,6 +791,15 @@ def main():
         "roofline": r["roofline"],
     }
     side = not args.only_main
+    if side and args.workload == "c1_sr_llama1b" and args.rng != "triton":
+        # the same workload with the reference's random-bit layout (one Philox block per
+        # element, tl.randint's), which is what a like-for-like reading of the kernel asks for
+        # (no empty_cache() before it: the allocator reuses the main run's blocks, and
+        # nothing is handed back to the driver while this is measured)
+        ref = time_adam_workload(args.workload, max(5, args.steps // 2), args.warmup, rng="triton")
+        out["roofline_reference_layout"] = dict(ref["roofline"], rng="triton")
+    torch.cuda.empty_cache()
+    progress(f"timed region done: {out['value']} GB/s, frac {out['roofline']['frac'] if out['roofline'] else None}")
     if side and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
         out["cpu_baseline"]["host"] = host_description()
@@ -694,6 +815,11 @@ def main():
             # default OffloadAdam, one micro-batch of 4096 tokens per step, with the check
             out["offloaded_step_1b"] = run_e2e(["--grad-accum", "1", "--check"], steps=10,
                                                warmup=3, timeout_s=200, model="llama1b")
+            out["mode_comparison_8b"] = mode_comparison_8b()
+            out["qat_step"] = qat_steps()
+    progress("done")
+    if side:
+        out["summary"] = summary_of(out)  # last key: it survives a log that keeps the tail
     print(json.dumps(out))
 
 

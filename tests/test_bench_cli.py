@@ -52,3 +52,51 @@ def test_cpu_baseline_fields_on_a_small_sample():
     assert "65536 elements" in row["sample"]
     host = bench.host_description()  # travels with the baseline in the bench line
     assert host["os_cpu_count"] >= 1 and host["numa_nodes"] >= 1 and host["torch_num_threads"] >= 1
+
+
+def test_summary_is_the_last_key_material_and_stays_small():
+    """``summary_of`` boils a full line down to what must survive a log that keeps
+    only the last 2000 characters."""
+    import json
+
+    import bench
+
+    roof = lambda f: {"frac": f, "achieved": 8000 * f}  # noqa: E731
+    step = {"step_s": 2.0123, "exposed_optimizer_s": 0.6123, "peak_gpu_GiB": 24.71,
+            "h2d_frac_of_bidir_peak": 0.831, "d2h_frac_of_bidir_peak": 0.829,
+            "check": {"passed": True}}
+    line = {
+        "roofline": roof(0.78), "roofline_reference_layout": roof(0.72),
+        "other_configs": {
+            "c0_fp32_master_16m": {"roofline": roof(0.73), "cache_assisted": {"roofline": roof(0.84)}},
+            "c2_fp31_clip_llama8b": {"adam_leg": {"roofline": roof(0.776)},
+                                     "norm_leg": {"roofline": roof(0.82)}},
+            "c3_codecs": {"kernels": [{"kernel": "quant_int8_kernel", "frac": 0.75},
+                                      {"kernel": "quant_int4_kernel", "frac": 0.67},
+                                      {"kernel": "dequant_nf4_kernel", "frac": 0.81},
+                                      {"kernel": "adam fp32_master + requant int8, fused", "frac": 0.66},
+                                      {"kernel": "adam fp32_master + requant int8, two moves",
+                                       "frac": 0.5}]},
+        },
+        "offloaded_step_8b": {"model": "x", "reference_traffic": step, "spare_hbm": step,
+                              "resident_adam": {"step_s": 1.47, "exposed_optimizer_s": 0.03,
+                                                "peak_gpu_GiB": 65.1},
+                              "clip_path_fp31": step},
+        "offloaded_step_1b": step,
+        "mode_comparison_8b": {"stochastic_rounding": step, "fp32_master": step},
+        "qat_step": {"llama1b": {k: step for k in ("none", "int8", "int4", "nf4", "nvfp4")},
+                     "llama8b": {"int4": {"error": "bench_e2e.py exited with 1"}}},
+    }
+    s = bench.summary_of(line)
+    assert s["frac"] == {"c1": 0.78, "c1_ref_bits": 0.72, "c0_cold": 0.73, "c0_cached": 0.84,
+                         "c2_step": 0.776, "c2_norm": 0.82, "c3_enc_min": 0.67,
+                         "c3_dec_min": 0.81, "c3_fused_min": 0.66}
+    assert s["steps"]["8b_ref"] == {"s": 2.0123, "exposed": 0.6123, "GiB": 24.71, "h2d": 0.831,
+                                    "d2h": 0.829, "ok": True}
+    assert "ok" not in s["steps"]["8b_adam"]
+    assert set(s["steps"]) == {"8b_ref", "8b_spare", "8b_adam", "8b_clip", "1b", "8b_ga1_sr",
+                               "8b_ga1_fp32m", "qat_1b_none", "qat_1b_int8", "qat_1b_int4",
+                               "qat_1b_nf4", "qat_1b_nvfp4", "qat_8b_int4"}
+    assert "error" in s["steps"]["qat_8b_int4"]
+    assert len(json.dumps({"summary": s})) < 1900
+    assert bench.summary_of({})["steps"] == {}
