@@ -758,8 +758,9 @@ quant_int4_kernel(const void* __restrict__ src, int64_t stride, int64_t rows, in
     }
   }
   __syncthreads();
-  if (full && (rows & 3) == 0) {
+  if (full && (rows & 3) == 0 && (reinterpret_cast<uintptr_t>(qweight) & 15) == 0) {
     // 16 bytes of the transposed payload per lane: four consecutive rows of one word column
+    // (a payload that is only 4-byte aligned takes the word-wise stores below)
     for (int idx = threadIdx.x; idx < wpr * (kI4RowsQ / 4); idx += kT) {
       const int kk = idx / (kI4RowsQ / 4), r4 = idx % (kI4RowsQ / 4);
       const u32x4 w = *reinterpret_cast<const u32x4*>(words + kk * kI4PitchQ + 4 * r4);

@@ -155,6 +155,55 @@ def test_strided_and_unaligned_sources(oracle):
         assert np.array_equal(s8.view(torch.uint8).cpu().numpy(), rs)
 
 
+def test_int4_payload_that_is_only_4_byte_aligned(oracle):
+    """A payload view 4, 8 or 12 bytes off a 16-byte boundary (row count a multiple of
+    four, whole tiles: the shape that otherwise takes the 16-byte transposed store) gets
+    the same words, from the plain encoder and from the fused step + re-encode."""
+    from offload_adam_amd import _lib
+    from offload_adam_amd.kernels import _common
+    from offload_adam_amd.qweight import _codec_ops as ops
+    from helpers import HYP, adam_inputs
+
+    rows, cols, group = 128, 512, 128
+    w = _weight(rows, cols, torch.float32, seed=6)
+    want_q, want_s = oracle.quant_int4(w.numpy(), group)
+    for off in (1, 2, 3):
+        buf = torch.zeros((cols // 8) * rows + 4, dtype=torch.int32, device="cuda")
+        qw = buf[off:off + (cols // 8) * rows].view(cols // 8, rows)
+        assert qw.data_ptr() % 16 == 4 * off
+        s = torch.empty(cols // group, rows, dtype=torch.bfloat16, device="cuda")
+        ops.quantize_int4_into(w.cuda(), group, qw, s)
+        assert np.array_equal(qw.cpu().numpy(), want_q), off
+        assert np.array_equal(_np_bits(s), _cast_scales(want_s, torch.bfloat16))
+        assert int(buf[:off].abs().sum()) == 0 and int(buf[off + (cols // 8) * rows:].abs().sum()) == 0
+    # fused step + re-encode through the C ABI into the same kind of view
+    _, st = adam_inputs(rows * cols, seed=8, mode="fp32_master", device="cuda")
+    ref = {k: v.clone() for k, v in st.items()}
+    b1h, b2h = _common.folded_betas(HYP["beta1"], HYP["beta2"], HYP["step"])
+    lib = _lib.load()
+
+    def fused(state, qw, s):
+        rc = lib.oa_adam_requant_int4(
+            _lib.ptr(state["grad"]), _lib.ptr(state["exp_avg"]), _lib.ptr(state["exp_avg_sq"]),
+            _lib.ptr(state["master_params"]), rows, cols, HYP["lr"], HYP["weight_decay"], b1h, b2h,
+            HYP["eps"], 1, None, group, _lib.ptr(qw), _lib.ptr(s), _lib.OA_BF16,
+            _lib.current_stream_ptr())
+        assert rc == 0
+
+    aligned = torch.empty(cols // 8, rows, dtype=torch.int32, device="cuda")
+    s0 = torch.empty(cols // group, rows, dtype=torch.bfloat16, device="cuda")
+    fused(ref, aligned, s0)
+    buf = torch.zeros((cols // 8) * rows + 4, dtype=torch.int32, device="cuda")
+    shifted = buf[1:1 + (cols // 8) * rows].view(cols // 8, rows)
+    s1 = torch.empty_like(s0)
+    fused(st, shifted, s1)
+    torch.cuda.synchronize()
+    assert torch.equal(shifted, aligned) and torch.equal(s1.view(torch.int16), s0.view(torch.int16))
+    assert torch.equal(st["master_params"], ref["master_params"])
+    master = ref["master_params"].cpu().numpy().reshape(rows, cols)
+    assert np.array_equal(aligned.cpu().numpy(), oracle.quant_int4(master, group)[0])
+
+
 def test_nf4_thresholds_match_brute_force(oracle):
     """The kernel's threshold count (bucket table) must equal the 16-way fp32
     distance search for every input: all floats within 64 ulps of each decision

@@ -61,6 +61,39 @@ def test_static_scratch_norm_matches_workspace_norm(oracle):
     assert torch.cuda.memory_allocated() == before
 
 
+def test_static_scratch_norm_takes_no_memory_from_the_driver():
+    """torch's allocator statistics cannot see a hipMalloc inside the library; the
+    driver's own count of free device memory can.  Batches of calls (after a first one,
+    which looks the array's address up) must leave it where it was."""
+    from offload_adam_amd import _lib
+
+    lib = _lib.load()
+    stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+    grads = [(torch.randn(n, generator=torch.Generator().manual_seed(n)) * 5e-3).to(BF16).cuda()
+             for n in (5_000_011, 300_001, 17)]
+    norm = torch.zeros(1, dtype=BF16, device="cuda")
+    sumsq = torch.zeros(1, dtype=torch.float32, device="cuda")
+
+    def call(g):
+        rc = lib.oa_grad_norm_bf16_static(c_void_p(g.data_ptr()), c_int64(g.numel()),
+                                          c_void_p(norm.data_ptr()), c_void_p(sumsq.data_ptr()),
+                                          stream)
+        assert rc == 0
+
+    for g in grads:
+        call(g)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    reserved_before = torch.cuda.memory_reserved()
+    for _ in range(50):
+        for g in grads:
+            call(g)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert torch.cuda.memory_reserved() == reserved_before  # torch itself took nothing either
+    assert free_after == free_before, (free_before, free_after)
+
+
 def test_static_scratch_norm_rejects_sizes_beyond_its_maximum():
     from offload_adam_amd import _lib
 
