@@ -582,7 +582,8 @@ def run_e2e(extra, steps, warmup, timeout_s, model="llama8b"):
             "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step", "d2h_GB_per_step",
             "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak", "link_floor_s", "pinned_GiB",
             "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB",
-            "peak_gpu_GiB", "optimizer_init_s", "copy_engines", "transfer_streams", "check",
+            "peak_gpu_GiB", "optimizer_init_s", "link_copies", "copy_engines", "transfer_streams",
+            "check",
             "max_grad_norm", "qat", "model_gpu_GiB", "pinned_limit",
             "loss_finite")
     row = {k: full[k] for k in keep if k in full}

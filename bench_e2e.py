@@ -229,6 +229,11 @@ class CopyTimeline:
         self.torch, self.oa_mod, self.log = torch, oa_mod, []
         self._orig = oa_mod._copy_async
         oa_mod._copy_async = self._timed_copy
+        # every copy its own library call, so that each can be bracketed by events (a
+        # stream round trip per copy: about 5 % slower than the batched default; under
+        # rocprofv3 --memory-copy-trace the default path itself is visible)
+        self._batched = oa_mod._BATCH_COPIES
+        oa_mod._BATCH_COPIES = False
 
     def _timed_copy(self, dst, src, kind, stream):
         e0 = self.torch.cuda.Event(enable_timing=True)
@@ -243,6 +248,7 @@ class CopyTimeline:
 
     def close(self):
         self.oa_mod._copy_async = self._orig
+        self.oa_mod._BATCH_COPIES = self._batched
 
     @staticmethod
     def _union(iv):
@@ -734,8 +740,13 @@ def run(args):
                                     (h2d + d2h) / 1e9 / (2 * peaks["bidir_each_GBps"])), 4)
     out["transfer_streams"] = opt.transfer_stream_report
     st = _copy_engines.status()
-    out["copy_engines"] = {k: st.get(k) for k in ("loaded", "active", "h2d_engine", "d2h_engine",
-                                                  "h2d_copies", "d2h_copies", "rejected")}
+    from offload_adam_amd import offload_adam as _oa_mod
+
+    out["link_copies"] = "direct" if _oa_mod._fixed_engine_copies() else "runtime"
+    out["copy_engines"] = {k: st.get(k) for k in (
+        "direct", "direct_reason", "direct_h2d_engine", "direct_d2h_engine", "direct_h2d_copies",
+        "direct_d2h_copies", "direct_runtime_copies", "loaded", "active", "h2d_copies",
+        "d2h_copies", "rejected")}
     if check is not None:
         check.before(opt)
         loop(opt, 1)
@@ -818,7 +829,13 @@ def main():
                          "occupancy per direction (adds two event records per copy)")
     ap.add_argument("--runtime-copy-engines", action="store_true",
                     help="leave the SDMA engine of each copy to the HIP runtime "
-                         "(do not load the fixed-engine tools library)")
+                         "(OFFLOAD_ADAM_COPY_ENGINES=off: neither the library's fixed-engine "
+                         "copies nor the tools library)")
+    ap.add_argument("--link-copies", default=None, choices=["direct", "runtime"],
+                    help="'direct': the kernel library issues the copies on its fixed engines "
+                         "(oa_link_copy_batch); 'runtime': hipMemcpyAsync, engine rewritten by "
+                         "the HSA tools library when it is loaded.  Default: 'runtime' when the "
+                         "tools library is in effect, else 'direct'")
     args = ap.parse_args()
     if args.qat:
         args.mode = "fp32_master"
@@ -826,6 +843,10 @@ def main():
         import os
 
         os.environ["OFFLOAD_ADAM_COPY_ENGINES"] = "off"  # before the package is imported
+    if args.link_copies:
+        import os
+
+        os.environ["OFFLOAD_ADAM_LINK_COPIES"] = args.link_copies
     if args.d2h_workgroups:
         from offload_adam_amd import offload_adam as _oa_mod
 

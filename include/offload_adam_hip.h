@@ -18,9 +18,10 @@
  *   - return value: 0 on success, a positive hipError_t from the HIP runtime,
  *     or a negative OA_E* code for an argument the library rejects; nothing is
  *     launched when the return value is non-zero;
- *   - re-entrant and never throws; no global mutable state, with one exception:
+ *   - re-entrant and never throws; no global mutable state, with two exceptions:
  *     oa_grad_norm_bf16_static keeps its partial sums in a device array inside
- *     the library (one per GPU) and caches that array's address per device.
+ *     the library (one per GPU) and caches that array's address per device, and
+ *     oa_h2d_async / oa_d2h_async keep a ring of signals per GPU.
  *
  * Element types: "bf16" = bfloat16 stored as uint16_t, "f32" = IEEE binary32,
  * "i16" = int16_t.  Scalars are binary32 because the reference's Triton
@@ -45,6 +46,8 @@ extern "C" {
 #define OA_EOVERLAP (-4) /* buffers that must be distinct alias each other */
 #define OA_EOS      (-5) /* an operating-system call failed; errno is reported
                             through the entry point's os_errno argument */
+#define OA_EUNAVAILABLE (-6) /* oa_h2d_async / oa_d2h_async: fixed-engine copies cannot be
+                                set up on this GPU; oa_link_copy_status says why */
 
 /* ABI version of the loaded library (== OA_ABI_VERSION it was built with). */
 int oa_abi_version(void);
@@ -394,6 +397,60 @@ int oa_gpu_numa_node(int device, int* node_out);
 #define OA_COPY_D2H 1
 #define OA_COPY_D2D 2
 int oa_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream);
+
+/* Host<->device copy of `bytes` on `stream`, on a fixed SDMA engine per direction.
+ * Stands in for the same calls as oa_memcpy_async (`host.to(device,
+ * non_blocking=True)` in OffloadAdam._issue_h2d, `host.copy_(dev, non_blocking=True)`
+ * in _issue_d2h, src/offload_adam/offload_adam.py:347-372) with the semantics of
+ * hipMemcpyAsync on `stream`: the copy starts after the work the stream was given
+ * before, work given afterwards starts after the copy.  What differs is who picks
+ * the SDMA engine: hipMemcpyAsync leaves it to the HIP runtime per copy (a saturated
+ * stream walks up to engines that run at a fifth of the link's rate, or onto the
+ * other direction's engine); here host->device copies always use one engine and
+ * device->host copies another (engines 0 and 1; OFFLOAD_ADAM_COPY_ENGINES="<h2d
+ * mask>,<d2h mask>" picks others, "off" disables the entry points).  The copy is
+ * handed to the ROCr runtime directly and fenced inside the stream with HIP's
+ * stream memory operations, so nothing depends on the process environment or on
+ * when the library was loaded, and profilers that trace HSA copies see it.
+ *   dst, src       one of them page-locked host memory, the other device memory
+ *   wait_event     NULL, or a hipEvent_t the stream waits for before the copy
+ *   record_event   NULL, or a hipEvent_t recorded on the stream after the copy
+ * Returns OA_EUNAVAILABLE, having enqueued nothing, when the GPU or the runtime
+ * lacks what this needs (the caller then uses oa_memcpy_async); a positive
+ * hipError_t when a HIP call fails.  Holds per-GPU state inside the library (a ring
+ * of 1024 signal pairs, set up at the first call on a GPU); safe to call from
+ * several threads; at most 1024 copies may be outstanding per GPU before a call
+ * waits for the oldest.  Not for use under stream capture. */
+int oa_h2d_async(void* dst, const void* src, size_t bytes, void* stream, void* wait_event,
+                 void* record_event);
+int oa_d2h_async(void* dst, const void* src, size_t bytes, void* stream, void* wait_event,
+                 void* record_event);
+
+/* `count` copies of one direction (kind = OA_COPY_H2D or OA_COPY_D2H) as one unit in
+ * the order of `stream` - what the loops over a parameter's states in
+ * OffloadAdam._issue_h2d / _issue_d2h (src/offload_adam/offload_adam.py:352-357,
+ * 366-371) amount to.  All of them start after the work the stream was given before
+ * the call; they run back to back on the direction's engine, without the stream
+ * coming round between two of them; the stream observes the completions in order
+ * and records record_events[i] (NULL array, or NULL entries, for none) behind copy
+ * i; work given to the stream after the call starts after the last copy.  Same
+ * availability, state and limits as oa_h2d_async. */
+int oa_link_copy_batch(int count, void* const* dsts, const void* const* srcs,
+                       const size_t* bytes, int kind, void* stream,
+                       void* const* record_events);
+
+/* State of the fixed-engine copies on the current GPU (sets them up if no copy has
+ * yet): 0 = in effect, else the reason they are not.  Any out pointer may be NULL:
+ * the engine masks in use, the copies issued per direction, and the copies the ROCr
+ * runtime declined, which went through hipMemcpyAsync instead. */
+#define OA_LINK_OFF                 (-10) /* OFFLOAD_ADAM_COPY_ENGINES=off */
+#define OA_LINK_NO_RUNTIME          (-11) /* libhsa-runtime64 or one of its entry points not found */
+#define OA_LINK_NO_STREAM_VALUE_OPS (-12) /* hipStreamWaitValue64 not supported by the device */
+#define OA_LINK_NO_AGENT            (-13) /* the HIP device was not found among the HSA agents */
+#define OA_LINK_NO_SIGNALS          (-14) /* signal memory could not be obtained or verified */
+int oa_link_copy_status(unsigned* h2d_engine, unsigned* d2h_engine,
+                        unsigned long long* h2d_copies, unsigned long long* d2h_copies,
+                        unsigned long long* runtime_copies);
 
 /* The same copy done by a small grid-stride kernel (`workgroups` blocks of 1024
  * lanes, 128-bit accesses, 4 loads in flight per lane; 8 blocks fill a PCIe

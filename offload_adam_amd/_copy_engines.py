@@ -85,12 +85,48 @@ def unregister_range(ptr):
         lib.oa_copy_engines_unregister_range(ctypes.c_void_p(ptr))
 
 
+def tools_loaded():
+    """True when the ROCr runtime has loaded the tools library (its OnLoad ran)."""
+    if not LIB_PATH.exists():
+        return False
+    lib = _lib()
+    lib.oa_copy_engines_loaded.restype = ctypes.c_int
+    lib.oa_copy_engines_active.restype = ctypes.c_int
+    return bool(lib.oa_copy_engines_loaded()) and bool(lib.oa_copy_engines_active())
+
+
+def direct_status():
+    """State of the kernel library's own fixed-engine copies (``oa_h2d_async`` /
+    ``oa_d2h_async``) on the current GPU: ``{"direct", "direct_reason",
+    "direct_h2d_engine", "direct_d2h_engine", "direct_h2d_copies", "direct_d2h_copies",
+    "direct_runtime_copies"}``.  Sets them up when no copy has been made yet (a GPU
+    call)."""
+    from . import _lib as kernels
+
+    lib = kernels.load()
+    h2d, d2h = ctypes.c_uint(0), ctypes.c_uint(0)
+    a, b, c = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
+    code = lib.oa_link_copy_status(ctypes.byref(h2d), ctypes.byref(d2h), ctypes.byref(a),
+                                   ctypes.byref(b), ctypes.byref(c))
+    return {"direct": code == 0,
+            "direct_reason": None if code == 0 else kernels.error_string(code),
+            "direct_h2d_engine": h2d.value, "direct_d2h_engine": d2h.value,
+            "direct_h2d_copies": a.value, "direct_d2h_copies": b.value,
+            "direct_runtime_copies": c.value}
+
+
 def status():
-    """What the tools library reports once the GPU runtime is up:
+    """Both ways of fixing the SDMA engine per direction.  The kernel library's own
+    copies: the keys of :func:`direct_status` (only once the GPU runtime is up; before
+    that ``direct`` is None).  The tools library, once the GPU runtime is up:
     ``{"install", "loaded", "active", "h2d_engine", "d2h_engine", "h2d_copies",
-    "d2h_copies", "rejected", "unpinned_calls", "scoped", "passed_by"}``.  ``loaded`` is False when the runtime started
-    before :func:`install` ran (or the library is missing)."""
-    out = {"install": _install_result, "loaded": False, "active": False}
+    "d2h_copies", "rejected", "unpinned_calls", "scoped", "passed_by"}``; ``loaded`` is
+    False when the runtime started before :func:`install` ran (or the library is
+    missing)."""
+    out = {"install": _install_result, "loaded": False, "active": False, "direct": None,
+           "direct_reason": "the GPU runtime has not started"}
+    if _gpu_runtime_started():
+        out.update(direct_status())
     if not LIB_PATH.exists():
         return out
     lib = _lib()

@@ -132,9 +132,22 @@ SIGNATURES = {
     "oa_gpu_numa_node": (c_int, [c_int, ctypes.POINTER(c_int)]),
     "oa_memcpy_async": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "oa_copy_kernel_async": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    # dst, src, bytes, stream, wait_event, record_event
+    "oa_h2d_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "oa_d2h_async": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),
+    # count, dsts, srcs, bytes, kind, stream, record_events
+    "oa_link_copy_batch": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                   c_void_p]),
+    "oa_link_copy_status": (
+        c_int,
+        [ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint),
+         ctypes.POINTER(ctypes.c_ulonglong), ctypes.POINTER(ctypes.c_ulonglong),
+         ctypes.POINTER(ctypes.c_ulonglong)],
+    ),
 }
 
 OA_EOS = -5
+OA_EUNAVAILABLE = -6
 OA_COPY_H2D, OA_COPY_D2H, OA_COPY_D2D = 0, 1, 2
 OA_F32, OA_BF16, OA_F16 = 0, 1, 2
 

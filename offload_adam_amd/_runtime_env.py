@@ -27,31 +27,18 @@ _prepared = None
 
 
 def required():
-    """True when ``OFFLOAD_ADAM_REQUIRE_COPY_ENGINES`` asks for an error instead of a
-    warning whenever the copy-engine library cannot take effect."""
+    """True when ``OFFLOAD_ADAM_REQUIRE_COPY_ENGINES`` asks ``OffloadAdam`` for an error
+    instead of a warning when its copies cannot be put on fixed SDMA engines."""
     return os.environ.get("OFFLOAD_ADAM_REQUIRE_COPY_ENGINES", "").strip().lower() in (
         "1", "on", "true", "yes")
 
 
-LATE_HINT = (
-    "offload_adam_amd was imported after the GPU runtime had started, so HSA_TOOLS_LIB and "
-    "GPU_MAX_HW_QUEUES come too late for this process: host<->device copies keep the SDMA "
-    "engine the HIP runtime picks and the streaming step runs half duplex.  Import "
-    "offload_adam_amd before the first CUDA call, start the script with "
-    "`python -m offload_adam_amd.launch script.py ...`, or export the variables first "
-    "(`python -m offload_adam_amd.launch --print-env`)."
-)
-
-
 def prepare():
-    """Idempotent; returns ``{"copy_engines": ..., "hw_queues": ...}``.  With
-    ``OFFLOAD_ADAM_REQUIRE_COPY_ENGINES=1`` an import that comes too late raises."""
+    """Idempotent; returns ``{"copy_engines": ..., "hw_queues": ...}``."""
     global _prepared
     if _prepared is not None:
         return _prepared
     result = {"copy_engines": _copy_engines.install()}
-    if result["copy_engines"] == "late" and required():
-        raise RuntimeError("OFFLOAD_ADAM_REQUIRE_COPY_ENGINES is set: " + LATE_HINT)
     want = os.environ.get("OFFLOAD_ADAM_HW_QUEUES", "").strip().lower()
     if want in ("off", "0", "none"):
         result["hw_queues"] = os.environ.get("GPU_MAX_HW_QUEUES")

@@ -23,10 +23,11 @@ What runs underneath is this package's HIP library: the fused AdamW kernels
 
 import bisect
 import operator
+import os
 import sys
 import time
 import warnings
-from ctypes import c_int, c_size_t, c_void_p
+from ctypes import c_int, c_size_t, c_uint64, c_void_p
 
 import torch
 from torch.optim.optimizer import Optimizer
@@ -56,14 +57,97 @@ def get_leaf_modules_with_params(module):
     return found
 
 
+# Who puts the optimizer's copies on fixed SDMA engines.  True: the kernel library's own
+# copies (oa_h2d_async / oa_d2h_async / oa_link_copy_batch).  False: hipMemcpyAsync, whose
+# engine the tools library rewrites when the ROCr runtime has loaded it.  None (default):
+# decided at the first copy - OFFLOAD_ADAM_LINK_COPIES=direct|runtime, else hipMemcpyAsync
+# when the tools library is in effect and the library's own copies when it is not (a
+# late import, a profiler attached).  The first is about 6 % faster on an 8B step (the
+# HIP runtime implements hipStreamWaitValue64 with a kernel that spins for the length of
+# the copy), the second needs nothing from the process environment.
+_FIXED_ENGINE_COPIES = None
+_fixed_engines_unavailable = set()  # device indices on which oa_h2d_async declined
+
+
+def _fixed_engine_copies():
+    global _FIXED_ENGINE_COPIES
+    if _FIXED_ENGINE_COPIES is None:
+        want = os.environ.get("OFFLOAD_ADAM_LINK_COPIES", "auto").strip().lower()
+        if want == "direct":
+            _FIXED_ENGINE_COPIES = True
+        elif want == "runtime":
+            _FIXED_ENGINE_COPIES = False
+        else:
+            _FIXED_ENGINE_COPIES = not _copy_engines.tools_loaded()
+    return _FIXED_ENGINE_COPIES
+
+
 def _copy_async(dst, src, kind, stream):
-    """hipMemcpyAsync (DMA engine) of a whole contiguous tensor on ``stream``."""
+    """Asynchronous copy of a whole contiguous tensor on ``stream`` by a DMA engine.
+
+    Host<->device copies go through ``oa_h2d_async`` / ``oa_d2h_async``: a fixed SDMA
+    engine per direction, chosen inside the library.  Where those are not available
+    (``OFFLOAD_ADAM_COPY_ENGINES=off``, a runtime without stream memory operations)
+    the copy is a ``hipMemcpyAsync`` and the HIP runtime picks the engine."""
     nbytes = src.numel() * src.element_size()
-    code = _lib.load().oa_memcpy_async(
+    lib = _lib.load()
+    if kind != _lib.OA_COPY_D2D and _fixed_engine_copies():
+        index = (dst if kind == _lib.OA_COPY_H2D else src).device.index
+        if index not in _fixed_engines_unavailable:
+            fn = lib.oa_h2d_async if kind == _lib.OA_COPY_H2D else lib.oa_d2h_async
+            code = fn(c_void_p(dst.data_ptr()), c_void_p(src.data_ptr()), c_size_t(nbytes),
+                      c_void_p(stream.cuda_stream), None, None)
+            if code != _lib.OA_EUNAVAILABLE:
+                _lib.check(code, "oa_h2d_async" if kind == _lib.OA_COPY_H2D else "oa_d2h_async")
+                return
+            _fixed_engines_unavailable.add(index)
+    code = lib.oa_memcpy_async(
         c_void_p(dst.data_ptr()), c_void_p(src.data_ptr()), c_size_t(nbytes), c_int(kind),
         c_void_p(stream.cuda_stream),
     )
     _lib.check(code, "oa_memcpy_async")
+
+
+_BATCH_COPIES = True  # False: one library call (and one stream round trip) per copy
+
+
+def _copy_batch(pairs, kind, stream, events=None):
+    """Copies ``pairs`` = [(dst, src), ...] of one direction on ``stream`` as one unit
+    (``oa_link_copy_batch``): they start after the work the stream has been given so
+    far and run back to back on the direction's engine.  ``events[i]``, when not None,
+    is a ``torch.cuda.Event`` that has been recorded before (so that it has a handle);
+    it is recorded again behind copy i.  Without the fixed-engine copies this is the
+    plain loop of ``_copy_async`` calls and event records."""
+    count = len(pairs)
+    if count == 0:
+        return
+    lib = _lib.load()
+    index = (pairs[0][0] if kind == _lib.OA_COPY_H2D else pairs[0][1]).device.index
+    if (_BATCH_COPIES and _fixed_engine_copies() and index not in _fixed_engines_unavailable):
+        dsts = (c_uint64 * count)(*[d.data_ptr() for d, _ in pairs])
+        srcs = (c_uint64 * count)(*[s.data_ptr() for _, s in pairs])
+        sizes = (c_size_t * count)(*[s.numel() * s.element_size() for _, s in pairs])
+        recs = None
+        if events is not None:
+            recs = (c_uint64 * count)(*[0 if e is None else e.cuda_event for e in events])
+        code = lib.oa_link_copy_batch(c_int(count), dsts, srcs, sizes, c_int(kind),
+                                      c_void_p(stream.cuda_stream), recs)
+        if code != _lib.OA_EUNAVAILABLE:
+            _lib.check(code, "oa_link_copy_batch")
+            return
+        _fixed_engines_unavailable.add(index)
+    for i, (dst, src) in enumerate(pairs):
+        _copy_async(dst, src, kind, stream)
+        if events is not None and events[i] is not None:
+            events[i].record(stream)
+
+
+def _handle_event(stream):
+    """A ``torch.cuda.Event`` with a handle the library can record (torch creates the
+    handle at the first record)."""
+    event = torch.cuda.Event()
+    event.record(stream)
+    return event
 
 
 _copy_engine_warned = False
@@ -744,29 +828,26 @@ class OffloadAdam(Optimizer):
     #   written again by the compute stream before that D2H is done.
 
     def _check_copy_engines(self):
-        """Warn once when the fixed-engine tools library is not in effect: the HIP
-        runtime then picks an SDMA engine per copy, and the streaming step runs
-        half duplex with stretches of 10 GB/s write-back."""
+        """Warn once when neither way of fixing the SDMA engine per direction is in
+        effect - the library's own copies (``oa_h2d_async`` / ``oa_d2h_async``) nor the
+        tools library that rewrites the HIP runtime's: the runtime then picks an engine
+        per copy, and the streaming step runs half duplex with stretches of 10 GB/s
+        write-back.  An error instead with ``OFFLOAD_ADAM_REQUIRE_COPY_ENGINES=1``."""
         global _copy_engine_warned
         st = _copy_engines.status()
-        if st["loaded"] or st["install"] == "off" or _copy_engine_warned:
+        if st["direct"] or st["loaded"] or st["install"] == "off":
             return
-        why = {
-            "late": "offload_adam_amd was imported after the GPU runtime had started",
-            "missing": f"{_copy_engines.LIB_PATH.name} is not built "
-                       "(python -m offload_adam_amd._build)",
-            "unusable_path": f"the path of {_copy_engines.LIB_PATH.name} contains whitespace, "
-                             "which HSA_TOOLS_LIB cannot name",
-        }.get(st["install"], "the ROCr runtime did not load it from HSA_TOOLS_LIB")
         message = (
-            "OffloadAdam: host<->device copies are not pinned to fixed SDMA engines ("
-            + why + "); expect a slower streaming step.  Import offload_adam_amd before "
-            "the first CUDA call, start the script with `python -m offload_adam_amd.launch`, "
-            "or set OFFLOAD_ADAM_COPY_ENGINES=off to silence this.")
+            "OffloadAdam: host<->device copies are not pinned to fixed SDMA engines (the "
+            f"library's own copies are unavailable: {st['direct_reason']}; "
+            f"{_copy_engines.LIB_PATH.name} is not in effect: {st['install']}); expect a slower "
+            "streaming step.  Set OFFLOAD_ADAM_COPY_ENGINES=off to silence this.")
         from . import _runtime_env
 
         if _runtime_env.required():
             raise RuntimeError("OFFLOAD_ADAM_REQUIRE_COPY_ENGINES is set: " + message)
+        if _copy_engine_warned:
+            return
         _copy_engine_warned = True
         warnings.warn(message, stacklevel=3)
 
@@ -809,20 +890,28 @@ class OffloadAdam(Optimizer):
                                torch.empty(host.shape, dtype=host.dtype, device=p.device)))
         h2d.wait_stream(self._compute_stream())
         last = len(staged) - 1
+        pairs, events = [], []
         for i, (p, key, host, buf) in enumerate(staged):
-            _copy_async(buf, host, _lib.OA_COPY_H2D, h2d)
+            pairs.append((buf, host))
             # the buffer belongs to the compute stream's pool: if it is dropped
             # before a consumer has waited for this copy, the allocator must not
             # hand it out again while the copy still writes it
             buf.record_stream(h2d)
             self.device_states[p][key] = buf
             if i == last or staged[i + 1][0] is not p:
-                self.h2d_events[p] = h2d.record_event()
+                # recorded again behind p's last copy by the batch below
+                events.append(_handle_event(h2d))
+                self.h2d_events[p] = events[-1]
+            else:
+                events.append(None)
+        # one unit: the engine runs the copies back to back, the stream follows
+        _copy_batch(pairs, _lib.OA_COPY_H2D, h2d, events)
 
     def _issue_d2h(self, p, keys):
         compute = self._compute_stream()
         dev = self.device_states[p]
         self.d2h_stream.wait_stream(compute)
+        pairs = []
         for key in keys:
             buf = dev[key]
             # Both directions use the DMA engines.  A copy kernel moves the same
@@ -833,10 +922,11 @@ class OffloadAdam(Optimizer):
             if _D2H_BY_KERNEL and buf.data_ptr() % 16 == 0:
                 _copy_by_kernel(self._host_view(p, key), buf, self.d2h_stream)
             else:
-                _copy_async(self._host_view(p, key), buf, _lib.OA_COPY_D2H, self.d2h_stream)
+                pairs.append((self._host_view(p, key), buf))
             buf.record_stream(self.d2h_stream)
             if not self._stays_on_device(p, key):
                 dev[key] = None
+        _copy_batch(pairs, _lib.OA_COPY_D2H, self.d2h_stream)
         self.d2h_events[p] = self.d2h_stream.record_event()
 
     def _stays_on_device(self, p, key):
@@ -850,14 +940,16 @@ class OffloadAdam(Optimizer):
             return
         d2h = self.d2h_stream
         d2h.wait_stream(self._compute_stream())
+        pairs = []
         for p, keys in items:
             dev = self.device_states[p]
             for key in keys:
                 buf = dev[key]
-                _copy_async(self._host_view(p, key), buf, _lib.OA_COPY_D2H, d2h)
+                pairs.append((self._host_view(p, key), buf))
                 buf.record_stream(d2h)
                 if not self._stays_on_device(p, key):
                     dev[key] = None
+        _copy_batch(pairs, _lib.OA_COPY_D2H, d2h)
         event = d2h.record_event()
         for p, _ in items:
             self.d2h_events[p] = event
