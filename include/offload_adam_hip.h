@@ -48,6 +48,8 @@ extern "C" {
                             through the entry point's os_errno argument */
 #define OA_EUNAVAILABLE (-6) /* oa_h2d_async / oa_d2h_async: fixed-engine copies cannot be
                                 set up on this GPU; oa_link_copy_status says why */
+#define OA_ELINKTIMEOUT (-7) /* a fixed-engine copy issued earlier had not completed after
+                                about a minute: its stream went on without it */
 
 /* ABI version of the loaded library (== OA_ABI_VERSION it was built with). */
 int oa_abi_version(void);
@@ -409,9 +411,10 @@ int oa_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* st
  * other direction's engine); here host->device copies always use one engine and
  * device->host copies another (engines 0 and 1; OFFLOAD_ADAM_COPY_ENGINES="<h2d
  * mask>,<d2h mask>" picks others, "off" disables the entry points).  The copy is
- * handed to the ROCr runtime directly and fenced inside the stream with HIP's
- * stream memory operations, so nothing depends on the process environment or on
- * when the library was loaded, and profilers that trace HSA copies see it.
+ * handed to the ROCr runtime directly and fenced inside the stream by two one-lane
+ * kernels (one releases the copy when the stream reaches it, one holds the stream
+ * until the engine has finished), so nothing depends on the process environment or
+ * on when the library was loaded, and profilers that trace HSA copies see it.
  *   dst, src       one of them page-locked host memory, the other device memory
  *   wait_event     NULL, or a hipEvent_t the stream waits for before the copy
  *   record_event   NULL, or a hipEvent_t recorded on the stream after the copy
@@ -445,7 +448,7 @@ int oa_link_copy_batch(int count, void* const* dsts, const void* const* srcs,
  * runtime declined, which went through hipMemcpyAsync instead. */
 #define OA_LINK_OFF                 (-10) /* OFFLOAD_ADAM_COPY_ENGINES=off */
 #define OA_LINK_NO_RUNTIME          (-11) /* libhsa-runtime64 or one of its entry points not found */
-#define OA_LINK_NO_STREAM_VALUE_OPS (-12) /* hipStreamWaitValue64 not supported by the device */
+#define OA_LINK_NO_STREAM_VALUE_OPS (-12) /* the device offers no signal memory (hipMallocSignalMemory) */
 #define OA_LINK_NO_AGENT            (-13) /* the HIP device was not found among the HSA agents */
 #define OA_LINK_NO_SIGNALS          (-14) /* signal memory could not be obtained or verified */
 int oa_link_copy_status(unsigned* h2d_engine, unsigned* d2h_engine,

@@ -10,26 +10,30 @@
 // (hsa_amd_memory_async_copy_on_engine), but an HSA copy is ordered by HSA signals
 // and a HIP stream does not hand its own out.
 //
-// How.  HIP's stream memory operations close the gap.  hipExtMallocWithFlags(...,
-// hipMallocSignalMemory) returns the value word of an HSA signal the HIP runtime
-// created (amd_signal_t, hsa/amd_hsa_signal.h: the signal's handle is the address of
-// that structure, its value the second 8-byte field; the library checks the
-// arithmetic against hsa_amd_signal_value_pointer for every signal it uses).  A
-// copy on stream S is then three asynchronous steps:
-//   1. hipStreamWriteValue64(S, dep, 0)        S reaches this point -> the copy may start
+// How.  hipExtMallocWithFlags(..., hipMallocSignalMemory) returns the value word of an
+// HSA signal the HIP runtime created, in host memory the GPU can address
+// (amd_signal_t, hsa/amd_hsa_signal.h: the signal's handle is the address of that
+// structure, its value the second 8-byte field; the library checks the arithmetic
+// against hsa_amd_signal_value_pointer for every signal it uses).  A copy on stream S
+// is then three asynchronous steps:
+//   1. link_release_kernel on S (dep := 0)     S reaches this point -> the copy may start
 //   2. hsa_amd_memory_async_copy_on_engine(..., dep, done, engine)
-//   3. hipStreamWaitValue64(S, done, == 0)     S goes on when the engine has finished
+//   3. link_wait_kernel on S (polls done)      S goes on when the engine has finished
 // so the copy starts after everything S was given before and everything S is given
 // afterwards starts after the copy: the semantics of hipMemcpyAsync on S.  Events
 // and cross-stream waits around it stay ordinary HIP calls.  Nothing here depends
 // on the process environment or on when the library was loaded, other streams'
-// copies are untouched, and a profiler that traces HSA copies sees these.
+// copies are untouched, and a profiler that traces HSA copies sees these.  (HIP's own
+// hipStreamWriteValue64 / hipStreamWaitValue64 are kernels too on this runtime; its
+// wait polls without pause, see link_wait_kernel.)  What it costs against a
+// hipMemcpyAsync whose engine is fixed from outside: the two one-lane kernels per
+// unit, about 4 % of an 8B training step that keeps both directions of the link busy.
 //
 // oa_link_copy_batch issues several copies of one direction as one unit: one
 // dependency signal for all of them (step 1 once), every copy handed to the engine
 // before the stream is given its first wait, then step 3 per copy - the engine runs
 // them back to back instead of waiting for the stream to come round between copies
-// (8B training step: 2.14 s with a round trip per copy, 2.0 s without).
+// and the stream runs one wait per recorded event instead of one per copy.
 //
 // Signals come from a ring per GPU; the slots of a unit are reused only after an
 // event recorded behind the unit's last wait has completed.  Not for use under stream
@@ -51,6 +55,32 @@
 #include "oa_common.hpp"
 
 namespace {
+
+// The stream-side wait for a copy: one lane polls the completion signal's value word
+// (host memory the engine decrements to 0) about every 3 us and returns when it reads
+// 0.  hipStreamWaitValue64 does the same with a kernel of the HIP runtime that polls
+// without pause; its reads cross the host link the copies are using, and an 8B
+// training step that streams 80 GB each way ran 6 % longer with it.  The wait is
+// bounded: after kMaxPolls (about a minute) the lane gives up, raises `*gave_up`
+// for the host to find, and the stream goes on - a copy that never completes must not
+// leave a wave spinning for good.
+constexpr unsigned kMaxPolls = 10u * 1000u * 1000u;
+
+__global__ void __launch_bounds__(64)
+link_wait_kernel(const int64_t* done, unsigned* gave_up) {
+  if (threadIdx.x != 0) return;
+  for (unsigned n = 0; n < kMaxPolls; ++n) {
+    if (__hip_atomic_load(done, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == 0) return;
+    __builtin_amdgcn_s_sleep(127);
+    __builtin_amdgcn_s_sleep(127);
+  }
+  __hip_atomic_store(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// The stream-side release of a unit's copies: writes 0 to the dependency signal.
+__global__ void __launch_bounds__(64) link_release_kernel(int64_t* dep) {
+  if (threadIdx.x == 0) __hip_atomic_store(dep, (int64_t)0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 struct HsaApi {
   decltype(hsa_init)* init = nullptr;
@@ -78,6 +108,7 @@ struct DeviceLink {
   hsa_agent_t gpu{}, cpu{};
   std::vector<Slot> ring;
   size_t next = 0;
+  unsigned* gave_up = nullptr;  // pinned host word a wait kernel raises when it times out
   std::atomic<unsigned long long> n_h2d{0}, n_d2h{0}, n_fallback{0};
 };
 
@@ -208,6 +239,13 @@ void set_up(DeviceLink& link, int dev) {
   if (g_hsa.agent_get_info(link.gpu, near_attr, &nearest) == HSA_STATUS_SUCCESS && nearest.handle)
     link.cpu = nearest;
 
+  if (hipHostMalloc(reinterpret_cast<void**>(&link.gave_up), sizeof(unsigned), hipHostMallocDefault) !=
+      hipSuccess) {
+    (void)hipGetLastError();
+    link.state = OA_LINK_NO_SIGNALS;
+    return;
+  }
+  *link.gave_up = 0;
   link.ring.resize(kRing);
   for (Slot& s : link.ring) {
     bool ok = hipExtMallocWithFlags(reinterpret_cast<void**>(&s.dep), 8, hipMallocSignalMemory) == hipSuccess &&
@@ -257,7 +295,8 @@ int issue_batch(DeviceLink& link, int count, void* const* dsts, const void* cons
   link.next = (first + count) % kRing;
   Slot& head = link.ring[first];
   g_hsa.signal_store(head.dep_sig, 1);
-  err = hipStreamWriteValue64(stream, head.dep, 0, 0);
+  hipLaunchKernelGGL(link_release_kernel, dim3(1), dim3(64), 0, stream, head.dep);
+  err = hipGetLastError();
   if (err != hipSuccess) return static_cast<int>(err);  // nothing else was enqueued
   const hsa_agent_t dst_agent = h2d ? link.gpu : link.cpu, src_agent = h2d ? link.cpu : link.gpu;
   const auto engine = static_cast<hsa_amd_sdma_engine_id_t>(h2d ? g_h2d_engine : g_d2h_engine);
@@ -271,12 +310,21 @@ int issue_batch(DeviceLink& link, int count, void* const* dsts, const void* cons
                              &head.dep_sig, s.done_sig, engine, false) != HSA_STATUS_SUCCESS)
       break;  // the runtime declined: this copy and the rest go through the HIP runtime
   }
+  // The engine completes a direction's copies in the order it was given them, so the
+  // stream only has to observe the copies something is recorded behind, and the last.
+  int last_taken = -1;
+  for (int i = 0; i < taken; ++i)
+    if (bytes[i] != 0) last_taken = i;
   int rc = 0;
   for (int i = 0; i < count && rc == 0; ++i) {
     Slot& s = link.ring[(first + i) % kRing];
     if (bytes[i] != 0) {
       if (i < taken) {
-        err = hipStreamWaitValue64(stream, s.done, 0, hipStreamWaitValueEq, ~0ull);
+        err = hipSuccess;
+        if (i == last_taken || (record_events && record_events[i])) {
+          hipLaunchKernelGGL(link_wait_kernel, dim3(1), dim3(64), 0, stream, s.done, link.gave_up);
+          err = hipGetLastError();
+        }
         (h2d ? link.n_h2d : link.n_d2h).fetch_add(1, std::memory_order_relaxed);
       } else {
         link.n_fallback.fetch_add(1, std::memory_order_relaxed);
@@ -312,6 +360,7 @@ int link_copies(int count, void* const* dsts, const void* const* srcs, const siz
   std::lock_guard<std::mutex> lock(link->mu);
   if (link->state == 0) set_up(*link, dev);
   if (link->state != 1) return OA_EUNAVAILABLE;
+  if (*static_cast<volatile unsigned*>(link->gave_up)) return OA_ELINKTIMEOUT;
   if (wait_event) {
     const hipError_t err = hipStreamWaitEvent(stream, static_cast<hipEvent_t>(wait_event), 0);
     if (err != hipSuccess) return static_cast<int>(err);
