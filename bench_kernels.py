@@ -5,7 +5,7 @@ the fused AdamW kernel with the clip coefficient folded in (fp31_master), and
 the eight weight codecs, and the fp32_master step of a quantised weight (fused
 with its re-encoding, and as the reference's two moves).  One JSON line per kernel.
 
-    python bench_kernels.py [--reps 20] [--only norm_large,norm_small,clip,adam,codecs,qat,stream]
+    python bench_kernels.py [--reps 20] [--only norm_large,norm_small,norm_multi,clip,adam,codecs,qat,stream]
 
 Shapes: the offloaded parameters of a Llama-3-8B-shaped decoder for the norm
 and AdamW kernels, one 4096 x 14336 bf16 weight ~N(0, 0.02) with 1 % outliers
@@ -87,6 +87,52 @@ def bench_norm_and_clip(args, torch, todo):
         coef = torch.ones((), dtype=torch.bfloat16, device="cuda")
         us = timed(lambda i: grad_clip.clip_coef_(per_param, 1.0, coef), args.reps, torch)
         line("clip_coef_kernel", "291 per-parameter norms", 2 * 291, us, bound="latency")
+
+
+def bench_norm_multi(args, torch):
+    """The 291 per-parameter norms of a Llama-3-8B-shaped model (16.06 GB of bf16
+    gradients) through the multi-tensor entry point: all in one call (9 pairs of
+    launches), grouped as OffloadAdam's hooks group them (36 gradients or 512 MB per
+    pair), and one call per gradient for comparison."""
+    import bench
+    from offload_adam_amd import grad_clip
+    from offload_adam_amd.offload_adam import OffloadAdam
+
+    shapes = bench.WORKLOADS["c2_fp31_clip_llama8b"]["shapes"]
+    g = torch.Generator(device="cuda").manual_seed(2)
+    grads = [(torch.randn(bench.numel(s), device="cuda", generator=g) * 3.35e-5).to(torch.bfloat16)
+             for _, s in shapes]
+    slots = torch.zeros(len(grads), dtype=torch.bfloat16, device="cuda")
+    views = [slots[i] for i in range(len(grads))]
+    nbytes = 2 * sum(t.numel() for t in grads)
+    groups, cur, cur_bytes = [], [], 0
+    for i, t in enumerate(grads):
+        cur.append(i)
+        cur_bytes += t.numel() * 2
+        if len(cur) >= grad_clip.NORMS_PER_LAUNCH or cur_bytes >= OffloadAdam._NORM_GROUP_BYTES:
+            groups.append(cur)
+            cur, cur_bytes = [], 0
+    if cur:
+        groups.append(cur)
+
+    def grouped(_):
+        for idx in groups:
+            grad_clip.grad_norms_([grads[i] for i in idx], [views[i] for i in idx], validate=False)
+
+    reps = max(3, args.reps // 8)
+    wl = "291 bf16 gradients of a Llama-3-8B-shaped model"
+    us = timed(lambda i: grad_clip.grad_norms_(grads, views, validate=False), reps, torch)
+    line("grad_norm_multi_partial_kernel + grad_norm_multi_final_kernel", wl + ", one call",
+         nbytes, us, launches=2 * -(-len(grads) // grad_clip.NORMS_PER_LAUNCH))
+    us = timed(grouped, reps, torch)
+    line("grad_norm_multi_partial_kernel + grad_norm_multi_final_kernel",
+         wl + f", {len(groups)} groups of up to 36 gradients or 512 MB", nbytes, us,
+         launches=2 * len(groups))
+    us = timed(lambda i: [grad_clip.grad_norm_(t, views[j]) for j, t in enumerate(grads)], reps,
+               torch)
+    line("grad_norm_partial_kernel + grad_norm_final_kernel", wl + ", one call per gradient",
+         nbytes, us, launches=sum(1 if t.numel() <= 16384 else 2 for t in grads),
+         note="host-bound: the launch rate of the Python loop")
 
 
 def bench_norm_large(args, torch, grad_clip):
@@ -260,9 +306,9 @@ def bench_qat_step(args, torch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=40)
-    ap.add_argument("--only", default="norm_large,norm_small,clip,adam,codecs,qat,stream",
-                    help="comma-separated subset of: norm_large, norm_small, clip, adam, codecs, "
-                         "qat, stream")
+    ap.add_argument("--only", default="norm_large,norm_small,norm_multi,clip,adam,codecs,qat,stream",
+                    help="comma-separated subset of: norm_large, norm_small, norm_multi, clip, adam, "
+                         "codecs, qat, stream")
     args = ap.parse_args()
 
     import torch
@@ -277,6 +323,8 @@ def main():
     todo = set(args.only.split(","))
     if todo & {"norm_large", "norm_small", "clip"}:
         bench_norm_and_clip(args, torch, todo)
+    if "norm_multi" in todo:
+        bench_norm_multi(args, torch)
     if "adam" in todo:
         bench_adam_clip(args, torch)
     if "codecs" in todo:
