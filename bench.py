@@ -33,6 +33,7 @@ After the timed region of the default workload the same line also carries
 """
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -340,18 +341,27 @@ def time_adam_workload(name, steps, warmup, *, rng=None, per_tensor=False, use_e
     # Timed region: exactly ``steps`` steps, bracketed by device synchronisation.
     # Events are recorded on the stream the kernels run on (torch's current
     # stream) and read back after the closing synchronisation.
+    # The collector is off inside it, as in timeit: a full collection of this process's
+    # heap takes about 80 ms, and one that falls between a start event and its launch
+    # turns a 20 ms measurement of 50 us launches into a quarter of its rate.
     pairs_per_step = 1 if multi else len(tensors)
     all_events = []
-    t0 = time.perf_counter()
-    for s in range(steps):
-        ev = None
-        if use_events:
-            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-                  for _ in range(pairs_per_step)]
-            all_events.append(ev)
-        one_step(warmup + s + 1, ev)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    gc.collect()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for s in range(steps):
+            ev = None
+            if use_events:
+                ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                      for _ in range(pairs_per_step)]
+                all_events.append(ev)
+            one_step(warmup + s + 1, ev)
+        enqueue = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    finally:
+        gc.enable()
     kernel_ms = sum(a.elapsed_time(b) for ev in all_events for a, b in ev)
     launches = launches_per_step * len(all_events)
 
@@ -379,6 +389,7 @@ def time_adam_workload(name, steps, warmup, *, rng=None, per_tensor=False, use_e
     return {
         "mode": mode, "tensors": len(tensors), "elements": total_elems,
         "bytes_per_step": bytes_per_step, "elapsed_s": elapsed, "roofline": roofline,
+        "host_enqueue_us_per_step": round(enqueue / steps * 1e6, 1),
         "launch": "multi_tensor" if multi else "per_tensor",
         "rng": (rng or "x8") if mode == "stochastic_rounding" else None,
     }
@@ -394,12 +405,11 @@ def config0_row(steps=400, warmup=20):
 
     row = {"workload": "fp32_master, one flat tensor of 16,777,216 elements, 20 B/elem",
            "floor_us_at_8TBps": 41.94}
-    # (the short same-operand run goes first: right after gigabytes of HBM are handed
-    # back, the driver's clearing of the freed pages competes with a 20 ms measurement)
     for label, sets in (("same_operands", 1), ("rotating_6_sets", 6)):
         r = time_adam_workload("c0_fp32_master_16m", steps, warmup, sets=sets)
         entry = {"ms_per_step": round(r["elapsed_s"] / steps * 1e3, 4),
                  "GBps_wall": round(r["bytes_per_step"] * steps / r["elapsed_s"] / 1e9, 1),
+                 "host_enqueue_us_per_step": r["host_enqueue_us_per_step"],
                  "roofline": r["roofline"]}
         if sets > 1:
             row["roofline"] = r["roofline"]
@@ -408,7 +418,6 @@ def config0_row(steps=400, warmup=20):
             entry["note"] = ("335 MB of operands reused every step; the 256 MiB memory-side "
                              "cache serves part of them")
             row["cache_assisted"] = entry
-        torch.cuda.empty_cache()
     return row
 
 
@@ -425,7 +434,6 @@ def config2_row(steps=5, warmup=2):
     row = {"adam_leg": {"ms_per_step": round(r["elapsed_s"] / steps * 1e3, 3),
                         "GBps_wall": round(r["bytes_per_step"] * steps / r["elapsed_s"] / 1e9, 1),
                         "roofline": r["roofline"], "floor_ms_at_8TBps": 18.07}}
-    torch.cuda.empty_cache()
     # norm leg: 291 gradients scaled so that the global norm is about 3
     dev = torch.device("cuda:0")
     shapes = WORKLOADS["c2_fp31_clip_llama8b"]["shapes"]
@@ -505,7 +513,6 @@ def config2_row(steps=5, warmup=2):
                 "torch.norm per parameter amounts to and is bound by the host's launch rate",
     }
     del grads
-    torch.cuda.empty_cache()
     row["workload"] = ("fp31_master + clip, Llama-3-8B shapes: 291 tensors, 8,030,261,248 "
                        "elements, norm 2 B/elem, step 18 B/elem")
     return row
@@ -523,11 +530,9 @@ def config3_row(reps=40):
     bench_kernels.SINK = rows = []
     try:
         bench_kernels.bench_codecs(args, torch)
-        torch.cuda.empty_cache()
         bench_kernels.bench_qat_step(args, torch)
     finally:
         bench_kernels.SINK = None
-    torch.cuda.empty_cache()
     keep = ("kernel", "alg_bytes_per_launch", "avg_launch_us", "achieved_GBps", "frac",
             "fused_speedup")
     return {"workload": "one 4096 x 14336 bf16 weight ~N(0, 0.02), 1 % of the entries x10",
@@ -795,11 +800,8 @@ def main():
     if side and args.workload == "c1_sr_llama1b" and args.rng != "triton":
         # the same workload with the reference's random-bit layout (one Philox block per
         # element, tl.randint's), which is what a like-for-like reading of the kernel asks for
-        # (no empty_cache() before it: the allocator reuses the main run's blocks, and
-        # nothing is handed back to the driver while this is measured)
         ref = time_adam_workload(args.workload, max(5, args.steps // 2), args.warmup, rng="triton")
         out["roofline_reference_layout"] = dict(ref["roofline"], rng="triton")
-    torch.cuda.empty_cache()
     progress(f"timed region done: {out['value']} GB/s, frac {out['roofline']['frac'] if out['roofline'] else None}")
     if side and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
@@ -811,6 +813,7 @@ def main():
         if not args.no_other_configs:
             out["other_configs"] = other_configs(cpu=not args.no_cpu_baseline)
         if not args.no_e2e:
+            torch.cuda.empty_cache()  # the child processes below need the HBM
             out["offloaded_step_8b"] = offloaded_step_8b()
             # benchmark config 1 as a training step: the 1.1B set streamed through the
             # default OffloadAdam, one micro-batch of 4096 tokens per step, with the check

@@ -18,6 +18,7 @@ events around ``--reps`` back-to-back launches on the launch stream / reps);
 """
 
 import argparse
+import gc
 import json
 import sys
 from pathlib import Path
@@ -41,11 +42,16 @@ def timed(fn, reps, torch):
         fn(i)
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    a.record()
-    for i in range(reps):
-        fn(i)
-    b.record()
-    torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()  # as timeit does: a full collection (about 80 ms here) would land in the interval
+    try:
+        a.record()
+        for i in range(reps):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+    finally:
+        gc.enable()
     return a.elapsed_time(b) / reps * 1e3
 
 

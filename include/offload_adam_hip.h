@@ -455,6 +455,17 @@ int oa_link_copy_status(unsigned* h2d_engine, unsigned* d2h_engine,
                         unsigned long long* h2d_copies, unsigned long long* d2h_copies,
                         unsigned long long* runtime_copies);
 
+/* Bound of the stream-side waits issued from now on on the current GPU, in polls of
+ * about 3 us each (0 = the default, about a minute; at most 2^32 - 1), and the way
+ * out of a timeout.  A wait that reaches its bound lets its stream go on with the
+ * copy still outstanding and marks the GPU's link: every later copy call returns
+ * OA_ELINKTIMEOUT, as does this call (after applying `max_polls`).  With
+ * `clear_timeout` non-zero the mark is taken off: only for a caller that has made
+ * sure, by its own means, that no copy is outstanding any more (the data of the copies
+ * issued since the timeout must be taken as undefined).  No counterpart in the
+ * reference (hipMemcpyAsync has no such bound). */
+int oa_link_wait_limit(unsigned long long max_polls, int clear_timeout);
+
 /* The same copy done by a small grid-stride kernel (`workgroups` blocks of 1024
  * lanes, 128-bit accesses, 4 loads in flight per lane; 8 blocks fill a PCIe
  * Gen5 x16 link) instead of the DMA engine.  Either pointer may be

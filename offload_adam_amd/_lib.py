@@ -138,6 +138,7 @@ SIGNATURES = {
     # count, dsts, srcs, bytes, kind, stream, record_events
     "oa_link_copy_batch": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                    c_void_p]),
+    "oa_link_wait_limit": (c_int, [ctypes.c_ulonglong, c_int]),
     "oa_link_copy_status": (
         c_int,
         [ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint),

@@ -61,15 +61,15 @@ namespace {
 // 0.  hipStreamWaitValue64 does the same with a kernel of the HIP runtime that polls
 // without pause; its reads cross the host link the copies are using, and an 8B
 // training step that streams 80 GB each way ran 6 % longer with it.  The wait is
-// bounded: after kMaxPolls (about a minute) the lane gives up, raises `*gave_up`
-// for the host to find, and the stream goes on - a copy that never completes must not
-// leave a wave spinning for good.
-constexpr unsigned kMaxPolls = 10u * 1000u * 1000u;
+// bounded: after `max_polls` (kDefaultPolls: about a minute) the lane gives up, raises
+// `*gave_up` for the host to find, and the stream goes on - a copy that never
+// completes must not leave a wave spinning for good.
+constexpr unsigned kDefaultPolls = 10u * 1000u * 1000u;
 
 __global__ void __launch_bounds__(64)
-link_wait_kernel(const int64_t* done, unsigned* gave_up) {
+link_wait_kernel(const int64_t* done, unsigned* gave_up, unsigned max_polls) {
   if (threadIdx.x != 0) return;
-  for (unsigned n = 0; n < kMaxPolls; ++n) {
+  for (unsigned n = 0; n < max_polls; ++n) {
     if (__hip_atomic_load(done, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == 0) return;
     __builtin_amdgcn_s_sleep(127);
     __builtin_amdgcn_s_sleep(127);
@@ -109,6 +109,7 @@ struct DeviceLink {
   std::vector<Slot> ring;
   size_t next = 0;
   unsigned* gave_up = nullptr;  // pinned host word a wait kernel raises when it times out
+  unsigned max_polls = kDefaultPolls;  // bound of the waits issued from now on
   std::atomic<unsigned long long> n_h2d{0}, n_d2h{0}, n_fallback{0};
 };
 
@@ -322,7 +323,8 @@ int issue_batch(DeviceLink& link, int count, void* const* dsts, const void* cons
       if (i < taken) {
         err = hipSuccess;
         if (i == last_taken || (record_events && record_events[i])) {
-          hipLaunchKernelGGL(link_wait_kernel, dim3(1), dim3(64), 0, stream, s.done, link.gave_up);
+          hipLaunchKernelGGL(link_wait_kernel, dim3(1), dim3(64), 0, stream, s.done, link.gave_up,
+                             link.max_polls);
           err = hipGetLastError();
         }
         (h2d ? link.n_h2d : link.n_d2h).fetch_add(1, std::memory_order_relaxed);
@@ -400,6 +402,20 @@ extern "C" int oa_link_copy_batch(int count, void* const* dsts, const void* cons
   if (kind != OA_COPY_H2D && kind != OA_COPY_D2H) return OA_EINVAL;
   return link_copies(count, dsts, srcs, bytes, kind == OA_COPY_H2D, stream, nullptr,
                      record_events);
+}
+
+extern "C" int oa_link_wait_limit(unsigned long long max_polls, int clear_timeout) {
+  if (max_polls > 0xFFFFFFFFull) return OA_ERANGE;
+  int dev = -1, rc = 0;
+  DeviceLink* link = current_link(&dev, &rc);
+  if (!link) return rc;
+  std::lock_guard<std::mutex> lock(link->mu);
+  if (link->state == 0) set_up(*link, dev);
+  if (link->state != 1) return OA_EUNAVAILABLE;
+  link->max_polls = max_polls ? static_cast<unsigned>(max_polls) : kDefaultPolls;
+  const bool timed_out = *static_cast<volatile unsigned*>(link->gave_up) != 0;
+  if (clear_timeout) *static_cast<volatile unsigned*>(link->gave_up) = 0;
+  return timed_out ? OA_ELINKTIMEOUT : 0;
 }
 
 extern "C" int oa_link_copy_status(unsigned* h2d_engine, unsigned* d2h_engine,

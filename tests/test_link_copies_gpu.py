@@ -263,3 +263,56 @@ def test_the_optimizer_uses_them_and_the_old_path_gives_the_same_bits(monkeypatc
     assert _status(lib)[3:5] == after[3:5]
     for a, b in zip(fixed, plain):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_bounded_wait_reports_a_copy_that_outlasts_it_and_recovers():
+    """The stream-side wait of a copy is bounded (``oa_link_wait_limit``): with a bound of
+    one poll and a 256 MB copy (about 5 ms on the link) the wait gives up while the
+    engine is still copying, the stream goes on, and every later copy call returns
+    OA_ELINKTIMEOUT until the caller clears the mark.  The condition is forced from the
+    host; every kernel involved exits by itself and the copy completes normally."""
+    from offload_adam_amd.pinned_alloc import zeros_pinned
+
+    kernels, lib = _lib()
+    OA_ELINKTIMEOUT = -7
+    rc = _status(lib)[0]
+    assert rc == 0, kernels.error_string(rc)
+    n = 64 << 20
+    host = zeros_pinned((n,), torch.int32, numa_node=None)
+    host.copy_(torch.arange(n, dtype=torch.int32))
+    dev = torch.zeros(n, dtype=torch.int32, device="cuda")
+    small_host = zeros_pinned((1024,), torch.int32, numa_node=None)
+    small_dev = torch.arange(1024, dtype=torch.int32, device="cuda")
+    s = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    assert lib.oa_link_wait_limit(1 << 40, 0) == -3  # OA_ERANGE: beyond 2^32 - 1
+    assert lib.oa_link_wait_limit(1, 0) == 0
+    try:
+        assert _h2d(lib, dev, host, s) == 0
+        assert _done(s, 10.0), "the bounded wait did not let the stream go on"
+        # the mark is up: nothing more is issued on this GPU's link
+        assert _d2h(lib, small_host, small_dev, s) == OA_ELINKTIMEOUT
+        assert lib.oa_link_wait_limit(0, 0) == OA_ELINKTIMEOUT
+        assert "time limit" in kernels.error_string(OA_ELINKTIMEOUT)
+        from offload_adam_amd import offload_adam as oa_mod
+
+        if oa_mod._fixed_engine_copies():
+            with pytest.raises(RuntimeError, match="time limit"):
+                oa_mod._copy_async(small_host, small_dev, kernels.OA_COPY_D2H, s)
+        # the copy itself was never lost: wait, by the clock, until all of it has landed
+        t0 = time.monotonic()
+        landed = False
+        while time.monotonic() - t0 < 20.0 and not landed:
+            time.sleep(0.05)
+            landed = bool((dev[-4096:].cpu() == host[-4096:]).all()) and int(dev[0].item()) == 0 \
+                and int(dev[n // 2].item()) == n // 2
+        assert landed
+        time.sleep(0.2)
+        assert torch.equal(dev.cpu(), host)
+    finally:
+        # (nothing is outstanding any more: the one copy issued under the mark has landed)
+        assert lib.oa_link_wait_limit(0, 1) in (0, OA_ELINKTIMEOUT)
+    assert lib.oa_link_wait_limit(0, 0) == 0
+    assert _d2h(lib, small_host, small_dev, s) == 0
+    assert _done(s)
+    assert torch.equal(small_host, small_dev.cpu())
