@@ -318,7 +318,11 @@ class OffloadAdam(Optimizer):
             the host link, no ``state[p]['grad']`` host buffer is allocated, and
             with ``grad_accum`` micro-batches the link traffic per step drops
             from ``2*(grad_accum-1)+4`` to ``4`` bytes per element each way in
-            ``stochastic_rounding`` mode.  Results are bit-identical.
+            ``stochastic_rounding`` mode.  Results are bit-identical, with one
+            exception: with ``max_grad_norm`` set, a parameter that received no
+            gradient since the last step sits ``step()`` out (the reference steps it
+            again from the old contents of its host gradient buffer, which does not
+            exist here).
         grad_cache_bytes (int | 'auto', keyword-only): with ``offload_grads=True``,
             HBM that may keep the device copy of accumulated gradients alive
             between micro-batches.  What is saved is fetching the same bytes again
@@ -1407,13 +1411,22 @@ class OffloadAdam(Optimizer):
         if self._step_in_backward:
             return
 
+        # A parameter whose gradient sum lives on the GPU only (offload_grads=False, or
+        # displaced by the pinned-memory limit) and that received no gradient in this
+        # window has nothing to be stepped with: it sits the step out, as on the hook
+        # path, and its norm does not count.  (With a host gradient buffer the reference
+        # steps such a parameter again with the buffer's old contents,
+        # src/offload_adam/offload_adam.py:446-454; that is kept where the buffer exists.)
+        idle = {p for p in self._grad_on_device if self.device_states[p].get("grad") is None}
         clip_coef = None
         if self.max_grad_norm is not None:
+            for p in idle:
+                self.state[p]["grad_norm"].zero_()
             grad_clip.clip_coef_(self._norm_slots, float(self.max_grad_norm), self._clip_coef,
                                  self._total_norm)
             clip_coef = self._clip_coef
 
-        order = [(g, p) for g in self.param_groups for p in g["params"]]
+        order = [(g, p) for g in self.param_groups for p in g["params"] if p not in idle]
         offloaded = [p for _, p in order if p not in self._inplace_params]
         ahead = 0  # offloaded params whose H2D has been issued
         done = 0

@@ -717,6 +717,49 @@ def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
     assert min(used) < steps and max(used) == steps  # some parameters did skip steps
 
 
+@pytest.mark.parametrize("kw", [dict(offload_grads=False), dict(pinned_limit_bytes=620_000)])
+def test_clip_path_leaves_out_parameters_whose_device_gradient_never_came(fixed_seed, kw):
+    """Clipping path, gradient sums kept on the GPU only: a parameter that got no gradient
+    in a window has no buffer to be stepped from; it sits the step out and its norm does
+    not count.  With weight_decay = 0 and modules that never run, the default optimizer
+    (host gradient buffers, all zero for those parameters: a step that changes nothing)
+    must give the same bits."""
+    from offload_adam_amd import OffloadAdam
+
+    steps, ga = 4, 2
+    data = batches(steps * ga)
+
+    def train(**extra):
+        torch.manual_seed(0)
+        model = BranchyNet().to(device="cuda", dtype=BF16)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            opt = OffloadAdam(model, mode="fp31_master", lr=1e-2, weight_decay=0.0,
+                              max_grad_norm=0.05, inplace_param_threshold=5000, **extra)
+        for s in range(steps):
+            for mb in range(ga):
+                opt.ready_for_optimizer_step = mb == ga - 1
+                out = model(data[s * ga + mb], route=1)  # block 1 and head2 never run
+                F.cross_entropy(out.float().reshape(-1, 50), data[s * ga + mb].reshape(-1)).backward()
+            opt.step()
+            opt.zero_grad()
+        torch.cuda.synchronize()
+        return model, opt
+
+    ref, _ = train()
+    got, opt = train(**kw)
+    assert_same_params(ref, got)
+    idle = [p for p in opt._grad_on_device if opt.state[p]["step"] == 0]
+    assert idle, "the case needs a parameter with its gradient on the GPU and no gradient"
+    assert any(opt.state[p]["step"] == steps for p in opt._grad_on_device)
+    torch.manual_seed(0)
+    fresh = BranchyNet().to(device="cuda", dtype=BF16)
+    names = {id(p): n for n, p in got.named_parameters()}
+    init = dict(fresh.named_parameters())
+    for p in idle:
+        assert torch.equal(p, init[names[id(p)]]), names[id(p)]
+
+
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("cache,policy", [(0, "write_back"), (40_000, "write_back"),
                                           (40_000, "write_through"), ("auto", "write_back"),
