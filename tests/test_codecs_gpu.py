@@ -125,6 +125,58 @@ def test_nvfp4(oracle, rows, cols, dtype):
         assert np.array_equal(_np_bits(got), _oracle_out_bits(want, odt)), odt
 
 
+@pytest.mark.parametrize("rows,cols", [(12288, 4096), (4096, 11008)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_large_shapes_of_the_reference_parity_tests(oracle, rows, cols, dtype):
+    """The two large shapes of the reference's parity lists (tests/test_int8.py:70-84,
+    tests/test_int4.py:91-116, tests/test_nf4.py:86-123, tests/test_nvfp4.py:98-134),
+    all four formats: codes, scales and the bf16 decode, bit for bit."""
+    from offload_adam_amd.qweight import _codec_ops as ops
+
+    w = _weight(rows, cols, dtype, seed=11)
+    src = w.float().numpy()
+    dev = w.cuda()
+    sdt = torch.bfloat16
+
+    q = torch.empty(rows, cols, dtype=torch.int8, device="cuda")
+    s = torch.empty(rows, dtype=sdt, device="cuda")
+    ops.quantize_int8_into(dev, q, s)
+    rq, rs = oracle.quant_int8(src)
+    assert np.array_equal(q.cpu().numpy(), rq)
+    assert np.array_equal(_np_bits(s), _cast_scales(rs, sdt))
+    want = oracle.dequant_int8(rq, s.float().cpu().numpy(), "bfloat16")
+    assert np.array_equal(_np_bits(ops.dequantize_int8(q, s, sdt)), want)
+
+    qw = torch.empty(cols // 8, rows, dtype=torch.int32, device="cuda")
+    s4 = torch.empty(cols // 128, rows, dtype=sdt, device="cuda")
+    ops.quantize_int4_into(dev, 128, qw, s4)
+    rq, rs = oracle.quant_int4(src, 128)
+    assert np.array_equal(qw.cpu().numpy(), rq)
+    assert np.array_equal(_np_bits(s4), _cast_scales(rs, sdt))
+    want = oracle.dequant_int4(rq, s4.float().cpu().numpy(), 128, "bfloat16")
+    assert np.array_equal(_np_bits(ops.dequantize_int4(qw, s4, 128, sdt)), want)
+
+    packed = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    absmax = torch.empty(rows * (cols // 64), dtype=torch.float32, device="cuda")
+    ops.quantize_nf4_into(dev, 64, packed, absmax)
+    rp, ra = oracle.quant_nf4(src, 64)
+    assert np.array_equal(absmax.cpu().numpy().view(np.uint32), ra.view(np.uint32))
+    assert np.array_equal(packed.cpu().numpy(), rp)
+    want = oracle.dequant_nf4(rp, ra, 64, "bfloat16")
+    assert np.array_equal(_np_bits(ops.dequantize_nf4(packed, absmax, cols, 64, sdt)), want)
+
+    pk4 = torch.empty(rows, cols // 2, dtype=torch.uint8, device="cuda")
+    s8 = torch.empty(rows, cols // 16, dtype=torch.float8_e4m3fn, device="cuda")
+    gs = torch.empty((), dtype=torch.float32, device="cuda")
+    ops.quantize_nvfp4_into(dev, pk4, s8, gs)
+    rp, rs, rgs = oracle.quant_nvfp4(src)
+    assert gs.cpu().numpy().view(np.uint32) == np.float32(rgs).view(np.uint32)
+    assert np.array_equal(s8.view(torch.uint8).cpu().numpy(), rs)
+    assert np.array_equal(pk4.cpu().numpy(), rp)
+    want = oracle.dequant_nvfp4(rp, rs, rgs, "bfloat16")
+    assert np.array_equal(_np_bits(ops.dequantize_nvfp4(pk4, s8, gs, cols, sdt)), want)
+
+
 def test_strided_and_unaligned_sources(oracle):
     """Column slices (row stride > cols) and views starting off a 16-byte
     boundary give the same codes as the contiguous copy."""
