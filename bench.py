@@ -343,10 +343,11 @@ def time_adam_workload(name, steps, warmup, *, rng=None, per_tensor=False, use_e
     # stream) and read back after the closing synchronisation.
     # The collector is off inside it, as in timeit: a full collection of this process's
     # heap takes about 80 ms, and one that falls between a start event and its launch
-    # turns a 20 ms measurement of 50 us launches into a quarter of its rate.
+    # turns a 20 ms measurement of 50 us launches into a quarter of its rate.  (Switched
+    # off only, not run first: collecting here would leave the GPU idle for those 80 ms
+    # between warm-up and measurement, and the clock-sensitive kernels then start slow.)
     pairs_per_step = 1 if multi else len(tensors)
     all_events = []
-    gc.collect()
     gc.disable()
     try:
         t0 = time.perf_counter()

@@ -42,7 +42,6 @@ def timed(fn, reps, torch):
         fn(i)
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    gc.collect()
     gc.disable()  # as timeit does: a full collection (about 80 ms here) would land in the interval
     try:
         a.record()
