@@ -647,7 +647,9 @@ def qat_steps():
     quantised, lm_head in bf16) through ``OffloadAdam`` as constructed by default,
     each followed by the numerical check of one more step: the four formats and the
     unquantised row on the 1.1B-shaped model, and int4 (the example's own command)
-    on the 8B-shaped one."""
+    on the 8B-shaped one; then the same five 1.1B rows with the GPU-resident ``Adam``
+    (no check there: tests/test_qat_replay_gpu.py replays that optimizer against the
+    oracle)."""
     common = ["--grad-accum", "1", "--seq", "8192", "--check"]
     rows = {"llama1b": {"none": run_e2e(common + ["--mode", "fp32_master"], steps=5, warmup=2,
                                         timeout_s=200, model="llama1b")}}
@@ -656,6 +658,13 @@ def qat_steps():
                                        model="llama1b")
     rows["llama8b"] = {"int4": run_e2e(common + ["--qat", "int4"], steps=3, warmup=1,
                                        timeout_s=300)}
+    # the table's other half: the GPU-resident Adam of this package on the same rows
+    resident = ["--grad-accum", "1", "--seq", "8192", "--optimizer", "adam"]
+    rows["llama1b_adam"] = {"none": run_e2e(resident + ["--mode", "fp32_master"], steps=5,
+                                            warmup=2, timeout_s=200, model="llama1b")}
+    for fmt in ("int8", "int4", "nf4", "nvfp4"):
+        rows["llama1b_adam"][fmt] = run_e2e(resident + ["--qat", fmt], steps=5, warmup=2,
+                                            timeout_s=200, model="llama1b")
     return rows
 
 

@@ -85,7 +85,10 @@ def test_summary_is_the_last_key_material_and_stays_small():
         "offloaded_step_1b": step,
         "mode_comparison_8b": {"stochastic_rounding": step, "fp32_master": step},
         "qat_step": {"llama1b": {k: step for k in ("none", "int8", "int4", "nf4", "nvfp4")},
-                     "llama8b": {"int4": {"error": "bench_e2e.py exited with 1"}}},
+                     "llama8b": {"int4": {"error": "bench_e2e.py exited with 1"}},
+                     "llama1b_adam": {k: {"step_s": 0.2123, "exposed_optimizer_s": 0.0123,
+                                          "peak_gpu_GiB": 12.34}
+                                      for k in ("none", "int8", "int4", "nf4", "nvfp4")}},
     }
     s = bench.summary_of(line)
     assert s["frac"] == {"c1": 0.78, "c1_ref_bits": 0.72, "c0_cold": 0.73, "c0_cached": 0.84,
@@ -96,7 +99,9 @@ def test_summary_is_the_last_key_material_and_stays_small():
     assert "ok" not in s["steps"]["8b_adam"]
     assert set(s["steps"]) == {"8b_ref", "8b_spare", "8b_adam", "8b_clip", "1b", "8b_ga1_sr",
                                "8b_ga1_fp32m", "qat_1b_none", "qat_1b_int8", "qat_1b_int4",
-                               "qat_1b_nf4", "qat_1b_nvfp4", "qat_8b_int4"}
+                               "qat_1b_nf4", "qat_1b_nvfp4", "qat_8b_int4", "qat_1b_adam_none",
+                               "qat_1b_adam_int8", "qat_1b_adam_int4", "qat_1b_adam_nf4",
+                               "qat_1b_adam_nvfp4"}
     assert "error" in s["steps"]["qat_8b_int4"]
-    assert len(json.dumps({"summary": s})) < 1900
+    assert len(json.dumps({"summary": s})) < 1950
     assert bench.summary_of({})["steps"] == {}
