@@ -95,7 +95,8 @@ struct Slot {
   int64_t* dep = nullptr;   // value words of two HIP-owned HSA signals
   int64_t* done = nullptr;
   hsa_signal_t dep_sig{}, done_sig{};
-  hipEvent_t passed = nullptr;  // recorded behind the slot's last use
+  hipEvent_t passed = nullptr;  // recorded behind a unit whose last slot this was
+  int fence = -1;  // slot whose `passed` event covers this slot's last use (its unit's last slot)
   bool used = false;
 };
 
@@ -286,8 +287,11 @@ int issue_batch(DeviceLink& link, int count, void* const* dsts, const void* cons
   for (int i = 0; i < count; ++i) {
     Slot& s = link.ring[(first + i) % kRing];
     if (s.used) {
-      // the stream that used this slot has passed its wait once this event is done
-      err = hipEventSynchronize(s.passed);
+      // The stream that used this slot is past the slot's unit once that unit's event is
+      // done.  (Slots are taken in ring order, so the event's own slot - the last of that
+      // unit - has not been handed out again, and the event not recorded again, before
+      // this one.)
+      err = hipEventSynchronize(link.ring[s.fence].passed);
       if (err != hipSuccess) return static_cast<int>(err);
       s.used = false;
     }
@@ -341,10 +345,19 @@ int issue_batch(DeviceLink& link, int count, void* const* dsts, const void* cons
     }
   }
   // The unit's signals (its one dependency signal above all) may be written again once
-  // the stream is past this point.
+  // the stream is past this point: one event for the unit, in its last slot.
+  const int fence = static_cast<int>((first + count - 1) % kRing);
+  const bool recorded = hipEventRecord(link.ring[fence].passed, stream) == hipSuccess;
+  if (!recorded && rc == 0) rc = static_cast<int>(hipGetLastError());
   for (int i = 0; i < count; ++i) {
     Slot& s = link.ring[(first + i) % kRing];
-    s.used = hipEventRecord(s.passed, stream) == hipSuccess;
+    s.fence = fence;
+    s.used = true;
+  }
+  if (!recorded) {
+    // without the event nothing tells when the slots are free again: wait here, once
+    (void)hipStreamSynchronize(stream);
+    for (int i = 0; i < count; ++i) link.ring[(first + i) % kRing].used = false;
   }
   return rc;
 }

@@ -111,6 +111,12 @@ def _copy_async(dst, src, kind, stream):
 _BATCH_COPIES = True  # False: one library call (and one stream round trip) per copy
 
 
+def _batched(device_index):
+    """Whether ``_copy_batch`` hands its copies to ``oa_link_copy_batch`` on this GPU."""
+    return (_BATCH_COPIES and _fixed_engine_copies()
+            and device_index not in _fixed_engines_unavailable)
+
+
 def _copy_batch(pairs, kind, stream, events=None):
     """Copies ``pairs`` = [(dst, src), ...] of one direction on ``stream`` as one unit
     (``oa_link_copy_batch``): they start after the work the stream has been given so
@@ -123,7 +129,7 @@ def _copy_batch(pairs, kind, stream, events=None):
         return
     lib = _lib.load()
     index = (pairs[0][0] if kind == _lib.OA_COPY_H2D else pairs[0][1]).device.index
-    if (_BATCH_COPIES and _fixed_engine_copies() and index not in _fixed_engines_unavailable):
+    if _batched(index):
         dsts = (c_uint64 * count)(*[d.data_ptr() for d, _ in pairs])
         srcs = (c_uint64 * count)(*[s.data_ptr() for _, s in pairs])
         sizes = (c_size_t * count)(*[s.numel() * s.element_size() for _, s in pairs])
@@ -587,6 +593,7 @@ class OffloadAdam(Optimizer):
         self._pending_writeback_bytes = 0
         self.device_states = {}
         self.h2d_events = {}
+        self._h2d_event_objs = {}  # library-issued copies: the event object each parameter keeps
         self.d2h_events = {}
         self._compute_streams = {}  # raw stream handle -> torch.cuda.Stream
         self.transfer_stream_report = None
@@ -894,18 +901,32 @@ class OffloadAdam(Optimizer):
                                torch.empty(host.shape, dtype=host.dtype, device=p.device)))
         h2d.wait_stream(self._compute_stream())
         last = len(staged) - 1
+        batched = _batched(staged[0][3].device.index)
         pairs, events = [], []
         for i, (p, key, host, buf) in enumerate(staged):
-            pairs.append((buf, host))
             # the buffer belongs to the compute stream's pool: if it is dropped
             # before a consumer has waited for this copy, the allocator must not
             # hand it out again while the copy still writes it
             buf.record_stream(h2d)
             self.device_states[p][key] = buf
-            if i == last or staged[i + 1][0] is not p:
-                # recorded again behind p's last copy by the batch below
-                events.append(_handle_event(h2d))
-                self.h2d_events[p] = events[-1]
+            last_of_p = i == last or staged[i + 1][0] is not p
+            if not batched:
+                _copy_async(buf, host, _lib.OA_COPY_H2D, h2d)
+                if last_of_p:
+                    self.h2d_events[p] = h2d.record_event()
+                continue
+            pairs.append((buf, host))
+            if last_of_p:
+                # One event object per parameter for good, recorded behind p's last copy
+                # by the batch below.  (It needs a handle, which torch creates at a first
+                # record; doing that once instead of before every batch keeps a marker
+                # per parameter and micro-batch out of the transfer stream.  A wait
+                # taken earlier keeps referring to the record it saw.)
+                event = self._h2d_event_objs.get(p)
+                if event is None:
+                    event = self._h2d_event_objs[p] = _handle_event(h2d)
+                events.append(event)
+                self.h2d_events[p] = event
             else:
                 events.append(None)
         # one unit: the engine runs the copies back to back, the stream follows
