@@ -588,7 +588,7 @@ def run_e2e(extra, steps, warmup, timeout_s, model="llama8b"):
             "fwd_bwd_only_s", "exposed_optimizer_s", "h2d_GB_per_step", "d2h_GB_per_step",
             "h2d_GBps_over_step", "d2h_GBps_over_step", "link_peak", "link_floor_s", "pinned_GiB",
             "prefetch_GiB", "grad_cache_GiB", "grad_cache_policy", "state_cache_GiB",
-            "peak_gpu_GiB", "optimizer_init_s", "link_copies", "copy_engines", "transfer_streams",
+            "peak_gpu_GiB", "peak_reserved_GiB", "fwd_bwd_only_reserved_GiB", "optimizer_init_s", "link_copies", "copy_engines", "transfer_streams",
             "check",
             "max_grad_norm", "qat", "model_gpu_GiB", "pinned_limit",
             "loss_finite")
@@ -668,12 +668,16 @@ def qat_steps():
     return rows
 
 
-def _step_summary(row):
-    """One streamed-step row boiled down for the summary at the end of the line."""
+def _step_summary(row, reserved=False):
+    """One streamed-step row boiled down for the summary at the end of the line
+    (``GiB``: peak HBM allocated, the reference's measure; ``res``: peak HBM the caching
+    allocator held from the driver)."""
     if not isinstance(row, dict) or "step_s" not in row:
         return {"error": (row or {}).get("error", "missing")[:60]} if isinstance(row, dict) else None
     out = {"s": row["step_s"], "exposed": row.get("exposed_optimizer_s"),
            "GiB": row.get("peak_gpu_GiB")}
+    if reserved and "peak_reserved_GiB" in row:
+        out["res"] = row["peak_reserved_GiB"]
     if "h2d_frac_of_bidir_peak" in row:
         out["h2d"], out["d2h"] = row["h2d_frac_of_bidir_peak"], row["d2h_frac_of_bidir_peak"]
     if "check" in row:
@@ -712,7 +716,7 @@ def summary_of(out):
     for key, name in (("reference_traffic", "8b_ref"), ("spare_hbm", "8b_spare"),
                       ("resident_adam", "8b_adam"), ("clip_path_fp31", "8b_clip")):
         if key in e8:
-            steps[name] = _step_summary(e8[key])
+            steps[name] = _step_summary(e8[key], reserved=True)
     if "offloaded_step_1b" in out:
         steps["1b"] = _step_summary(out["offloaded_step_1b"])
     for key, row in out.get("mode_comparison_8b", {}).items():

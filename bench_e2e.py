@@ -675,7 +675,10 @@ def run(args):
 
     # 1) forward/backward only: what a step costs with a free optimizer
     loop(None, 1)
+    torch.cuda.reset_peak_memory_stats()
     out["fwd_bwd_only_s"] = round(loop(None, args.steps), 4)
+    out["fwd_bwd_only_peak_GiB"] = round(torch.cuda.max_memory_allocated() / 1024**3, 2)
+    out["fwd_bwd_only_reserved_GiB"] = round(torch.cuda.max_memory_reserved() / 1024**3, 2)
 
     if args.optimizer == "adam":
         return run_resident_adam(args, out, model, loop, torch)
@@ -713,6 +716,8 @@ def run(args):
         from offload_adam_amd import offload_adam as oa_mod
 
         timeline = CopyTimeline(torch, oa_mod)
+    model.zero_grad(set_to_none=True)
+    torch.cuda.empty_cache()  # so that the reserved figure below is this phase's own
     torch.cuda.reset_peak_memory_stats()
     loop(opt, args.warmup)
     if timeline:
@@ -728,6 +733,13 @@ def run(args):
     out["tokens_per_s"] = round(args.grad_accum * args.seq / step_s, 1)
     out["exposed_optimizer_s"] = round(step_s - out["fwd_bwd_only_s"], 4)
     out["peak_gpu_GiB"] = round(torch.cuda.max_memory_allocated() / 1024**3, 2)
+    # what the caching allocator holds from the driver: includes blocks that were freed
+    # but wait for a copy on another stream (record_stream) before they can be reused
+    out["peak_reserved_GiB"] = round(torch.cuda.max_memory_reserved() / 1024**3, 2)
+    stats = torch.cuda.memory_stats()
+    out["allocator"] = {"device_allocs": stats.get("num_device_alloc"),
+                        "device_frees": stats.get("num_device_free"),
+                        "alloc_retries": stats.get("num_alloc_retries")}
     h2d, d2h = link_bytes_per_step(opt, args.grad_accum)
     out["h2d_GB_per_step"] = round(h2d / 1e9, 2)
     out["d2h_GB_per_step"] = round(d2h / 1e9, 2)
@@ -791,6 +803,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--d2h-workgroups", type=int, default=None,
                     help="workgroups of the write-back copy kernel (default: the optimizer's)")
+    ap.add_argument("--writeback-pending-gib", type=float, default=None,
+                    help="bytes of freed staging buffers that write-backs may still be reading "
+                         "before the host waits (default: the optimizer's, = its staging window)")
     ap.add_argument("--prefetch-gib", type=float, default=None,
                     help="device staging budget of the H2D prefetch window")
     ap.add_argument("--optimizer", default="offload", choices=["offload", "adam"],
@@ -852,6 +867,10 @@ def main():
 
         _oa_mod._D2H_BY_KERNEL = True
         _oa_mod._D2H_WORKGROUPS = args.d2h_workgroups
+    if args.writeback_pending_gib is not None:
+        from offload_adam_amd import OffloadAdam as _OffloadAdam
+
+        _OffloadAdam._WRITEBACK_PENDING_BYTES = int(args.writeback_pending_gib * 2**30)
     print(json.dumps(run(args)))
 
 

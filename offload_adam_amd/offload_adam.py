@@ -22,6 +22,7 @@ What runs underneath is this package's HIP library: the fused AdamW kernels
 """
 
 import bisect
+import collections
 import operator
 import os
 import sys
@@ -309,7 +310,11 @@ class OffloadAdam(Optimizer):
             ``grad_cache_policy`` becomes ``'write_back'``.  The HBM that may be
             held is printed once at construction.  Results are bit-identical.
         prefetch_bytes (int | 'auto', keyword-only): device staging the hook path
-            may fill ahead of the gradient hooks.  Default 4 GiB (and never fewer
+            may fill ahead of the gradient hooks (the same number of bytes, twice
+            that with ``max_grad_norm``, bounds the staging buffers that have been
+            handed back while their write-back is still running: beyond it the host
+            waits for the oldest write-back, which keeps the HBM really held close
+            to the HBM allocated).  Default 4 GiB (and never fewer
             than the next two parameters); ``'auto'``: a tenth of the HBM that is
             free when the optimizer is built, at least 2 GiB.  The copies of a
             parameter's states start this far ahead in backward order; once a
@@ -395,6 +400,7 @@ class OffloadAdam(Optimizer):
     # the offloaded bytes when that is less (a 1B-parameter model steps 3 % faster with
     # 0.75 GiB than with 4, at a third less HBM: its write-backs have the link to themselves)
     _PREFETCH_BYTES = 4 << 30
+    _WRITEBACK_PENDING_BYTES = None  # None: derived from the staging window, see __init__
     _PREFETCH_BYTES_MIN = 256 << 20
 
     def __init__(
@@ -592,6 +598,21 @@ class OffloadAdam(Optimizer):
         self._pending_writebacks = []  # cached gradients whose write-back waits for its group
         self._pending_writeback_bytes = 0
         self.device_states = {}
+        # Device buffers given back to the allocator while a write-back still reads them
+        # (``record_stream``): they no longer count as allocated, yet their memory is in
+        # use until the copy is done.  The hooks run as fast as the host can enqueue, far
+        # ahead of the link, so without a bound every staged byte of a pass ends up in
+        # that state at once (8B model: 61 GiB held from the driver at 24.7 GiB
+        # "allocated"; 96 GiB on the clipping path).  ``_throttle_writebacks`` makes the
+        # host wait for the oldest write-back once more than this many bytes are pending.
+        self._writebacks_pending = collections.deque()  # (event, bytes), write-back order
+        self._writeback_pending_bytes = 0
+        # Measured free of charge (8B and 1.1B steps): the staging window on the hook
+        # path, twice that on the clipping path (whose step() is link-bound from end to
+        # end), and never less than 2 GiB; half of it costs 3-6 %.
+        self._writeback_pending_limit = (
+            self._WRITEBACK_PENDING_BYTES if self._WRITEBACK_PENDING_BYTES is not None
+            else max(self._PREFETCH_BYTES * (1 if self._step_in_backward else 2), 2 << 30))
         self.h2d_events = {}
         self._h2d_event_objs = {}  # library-issued copies: the event object each parameter keeps
         self.d2h_events = {}
@@ -889,6 +910,7 @@ class OffloadAdam(Optimizer):
         previous users of its buffer."""
         if not items:
             return
+        self._throttle_writebacks()  # before more staging is allocated
         h2d = self.h2d_stream
         staged = []
         for p, keys in items:
@@ -932,11 +954,29 @@ class OffloadAdam(Optimizer):
         # one unit: the engine runs the copies back to back, the stream follows
         _copy_batch(pairs, _lib.OA_COPY_H2D, h2d, events)
 
+    def _throttle_writebacks(self):
+        """Keep the bytes that freed staging buffers still occupy below the limit: forget
+        write-backs that have completed, then wait (the host, not a stream) for the
+        oldest ones until the rest fits."""
+        pending = self._writebacks_pending
+        while pending and pending[0][0].query():
+            self._writeback_pending_bytes -= pending.popleft()[1]
+        while pending and self._writeback_pending_bytes > self._writeback_pending_limit:
+            event, nbytes = pending.popleft()
+            event.synchronize()
+            self._writeback_pending_bytes -= nbytes
+
+    def _note_writeback(self, event, nbytes):
+        if nbytes:
+            self._writebacks_pending.append((event, nbytes))
+            self._writeback_pending_bytes += nbytes
+
     def _issue_d2h(self, p, keys):
+        self._throttle_writebacks()
         compute = self._compute_stream()
         dev = self.device_states[p]
         self.d2h_stream.wait_stream(compute)
-        pairs = []
+        pairs, released = [], 0
         for key in keys:
             buf = dev[key]
             # Both directions use the DMA engines.  A copy kernel moves the same
@@ -951,8 +991,10 @@ class OffloadAdam(Optimizer):
             buf.record_stream(self.d2h_stream)
             if not self._stays_on_device(p, key):
                 dev[key] = None
+                released += buf.numel() * buf.element_size()
         _copy_batch(pairs, _lib.OA_COPY_D2H, self.d2h_stream)
-        self.d2h_events[p] = self.d2h_stream.record_event()
+        event = self.d2h_events[p] = self.d2h_stream.record_event()
+        self._note_writeback(event, released)
 
     def _stays_on_device(self, p, key):
         """Write-through caches: the device copy outlives its write-back."""
@@ -963,9 +1005,10 @@ class OffloadAdam(Optimizer):
         event for the group (a later fetch of any of them waits for all)."""
         if not items:
             return
+        self._throttle_writebacks()
         d2h = self.d2h_stream
         d2h.wait_stream(self._compute_stream())
-        pairs = []
+        pairs, released = [], 0
         for p, keys in items:
             dev = self.device_states[p]
             for key in keys:
@@ -974,10 +1017,12 @@ class OffloadAdam(Optimizer):
                 buf.record_stream(d2h)
                 if not self._stays_on_device(p, key):
                     dev[key] = None
+                    released += buf.numel() * buf.element_size()
         _copy_batch(pairs, _lib.OA_COPY_D2H, d2h)
         event = d2h.record_event()
         for p, _ in items:
             self.d2h_events[p] = event
+        self._note_writeback(event, released)
 
     def _ensure_on_device(self, p, keys):
         dev = self.device_states[p]
@@ -1597,6 +1642,8 @@ class OffloadAdam(Optimizer):
                 dev[name] = None
         self.h2d_events.clear()
         self.d2h_events.clear()
+        self._writebacks_pending.clear()  # (after the synchronisation above)
+        self._writeback_pending_bytes = 0
         self._stale_host_grads.clear()
         self._bw_cursor = -1
         self._bw_issued_upto = 0

@@ -63,6 +63,7 @@ def test_summary_is_the_last_key_material_and_stays_small():
 
     roof = lambda f: {"frac": f, "achieved": 8000 * f}  # noqa: E731
     step = {"step_s": 2.0123, "exposed_optimizer_s": 0.6123, "peak_gpu_GiB": 24.71,
+            "peak_reserved_GiB": 39.81,
             "h2d_frac_of_bidir_peak": 0.831, "d2h_frac_of_bidir_peak": 0.829,
             "check": {"passed": True}}
     line = {
@@ -94,8 +95,9 @@ def test_summary_is_the_last_key_material_and_stays_small():
     assert s["frac"] == {"c1": 0.78, "c1_ref_bits": 0.72, "c0_cold": 0.73, "c0_cached": 0.84,
                          "c2_step": 0.776, "c2_norm": 0.82, "c3_enc_min": 0.67,
                          "c3_dec_min": 0.81, "c3_fused_min": 0.66}
-    assert s["steps"]["8b_ref"] == {"s": 2.0123, "exposed": 0.6123, "GiB": 24.71, "h2d": 0.831,
-                                    "d2h": 0.829, "ok": True}
+    assert s["steps"]["8b_ref"] == {"s": 2.0123, "exposed": 0.6123, "GiB": 24.71, "res": 39.81,
+                                    "h2d": 0.831, "d2h": 0.829, "ok": True}
+    assert "res" not in s["steps"]["1b"]
     assert "ok" not in s["steps"]["8b_adam"]
     assert set(s["steps"]) == {"8b_ref", "8b_spare", "8b_adam", "8b_clip", "1b", "8b_ga1_sr",
                                "8b_ga1_fp32m", "qat_1b_none", "qat_1b_int8", "qat_1b_int4",

@@ -717,6 +717,35 @@ def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
     assert min(used) < steps and max(used) == steps  # some parameters did skip steps
 
 
+@pytest.mark.parametrize("mode,clip", [("stochastic_rounding", None), ("fp31_master", 0.05),
+                                       ("fp32_master", None)])
+def test_bound_on_pending_write_backs_changes_no_result(fixed_seed, mode, clip, monkeypatch):
+    """Staging buffers handed back while their write-back still runs are bounded in bytes;
+    past the bound the host waits for the oldest write-back.  With a bound of one byte
+    (a wait at every issue) and with none, on the hook path and the clipping path: the
+    same bits, and the books are back at zero once everything has completed."""
+    from offload_adam_amd import OffloadAdam
+
+    results = []
+    for limit in (1, 1 << 60):
+        monkeypatch.setattr(OffloadAdam, "_WRITEBACK_PENDING_BYTES", limit)
+        model, opt = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip)
+        assert opt._writeback_pending_limit == limit
+        if limit == 1:
+            # nothing older than the newest write-back is ever left pending
+            assert len(opt._writebacks_pending) <= 1
+        else:
+            assert opt._writeback_pending_bytes > 0  # (the last ones were never waited for)
+        torch.cuda.synchronize()
+        opt._throttle_writebacks()
+        assert opt._writeback_pending_bytes == 0 and not opt._writebacks_pending
+        results.append(model)
+    assert_same_params(results[0], results[1])
+    if clip is None:
+        ref, _ = run_reference_adam(mode, steps=3, ga=3)
+        assert_same_params(ref, results[0])
+
+
 @pytest.mark.parametrize("kw", [dict(offload_grads=False), dict(pinned_limit_bytes=620_000)])
 def test_clip_path_leaves_out_parameters_whose_device_gradient_never_came(fixed_seed, kw):
     """Clipping path, gradient sums kept on the GPU only: a parameter that got no gradient
