@@ -310,11 +310,10 @@ class OffloadAdam(Optimizer):
             ``grad_cache_policy`` becomes ``'write_back'``.  The HBM that may be
             held is printed once at construction.  Results are bit-identical.
         prefetch_bytes (int | 'auto', keyword-only): device staging the hook path
-            may fill ahead of the gradient hooks (the same number of bytes, twice
-            that with ``max_grad_norm``, bounds the staging buffers that have been
-            handed back while their write-back is still running: beyond it the host
-            waits for the oldest write-back, which keeps the HBM really held close
-            to the HBM allocated).  Default 4 GiB (and never fewer
+            may fill ahead of the gradient hooks (twice that number of bytes bounds
+            the staging buffers that have been handed back while their write-back
+            is still running: beyond it the host waits for the oldest write-back,
+            which keeps the HBM really held close to the HBM allocated).  Default 4 GiB (and never fewer
             than the next two parameters); ``'auto'``: a tenth of the HBM that is
             free when the optimizer is built, at least 2 GiB.  The copies of a
             parameter's states start this far ahead in backward order; once a
@@ -374,6 +373,16 @@ class OffloadAdam(Optimizer):
             below ``inplace_param_threshold``).  One notice on stderr says what
             was moved; ``RuntimeError`` only when HBM cannot take it either.
             Results are bit-identical.
+        pending_writeback_bytes (int | None, keyword-only): bytes of staging buffers
+            that may be handed back to the allocator while their write-back to the
+            host is still running.  Such memory no longer counts as allocated but
+            is not free either, and the hooks run far ahead of the host link; past
+            this limit the host waits for the oldest write-back before it stages
+            more.  ``None`` (default): twice the staging window (``prefetch_bytes``),
+            at least 2 GiB - free of charge where micro-batches are accumulated and
+            with ``max_grad_norm``, 0.6-2 % on steps of one micro-batch, which a
+            limit of four windows avoids at that much more HBM held.  Results are
+            bit-identical.
     """
 
     supported_modes = {
@@ -425,6 +434,7 @@ class OffloadAdam(Optimizer):
         grad_cache_policy=None,
         spare_hbm=False,
         pinned_limit_bytes=None,
+        pending_writeback_bytes=None,
     ):
         if prefetch_policy not in ("eager", "lazy"):
             raise ValueError(f"prefetch_policy must be 'eager' or 'lazy' (got {prefetch_policy!r})")
@@ -461,6 +471,10 @@ class OffloadAdam(Optimizer):
         grad_cache_bytes = byte_count("grad_cache_bytes", grad_cache_bytes)
         state_cache_bytes = byte_count("state_cache_bytes", state_cache_bytes)
         self._pinned_limit_arg = byte_count("pinned_limit_bytes", pinned_limit_bytes, auto_ok=False)
+        pending_writeback_bytes = byte_count("pending_writeback_bytes", pending_writeback_bytes,
+                                             auto_ok=False)
+        if pending_writeback_bytes is not None:
+            self._WRITEBACK_PENDING_BYTES = pending_writeback_bytes
         self.spare_hbm = bool(spare_hbm)
         if self.spare_hbm:
             prefetch_bytes = "auto" if prefetch_bytes is None else prefetch_bytes
@@ -607,12 +621,13 @@ class OffloadAdam(Optimizer):
         # host wait for the oldest write-back once more than this many bytes are pending.
         self._writebacks_pending = collections.deque()  # (event, bytes), write-back order
         self._writeback_pending_bytes = 0
-        # Measured free of charge (8B and 1.1B steps): the staging window on the hook
-        # path, twice that on the clipping path (whose step() is link-bound from end to
-        # end), and never less than 2 GiB; half of it costs 3-6 %.
+        # Twice the staging window, at least 2 GiB: free of charge where micro-batches
+        # are accumulated and on the clipping path, at most 2 % on steps of a single
+        # micro-batch (link-bound from end to end, where the host's lead over the link is
+        # what keeps both directions busy); the window itself costs those 5-10 %.
         self._writeback_pending_limit = (
             self._WRITEBACK_PENDING_BYTES if self._WRITEBACK_PENDING_BYTES is not None
-            else max(self._PREFETCH_BYTES * (1 if self._step_in_backward else 2), 2 << 30))
+            else max(2 * self._PREFETCH_BYTES, 2 << 30))
         self.h2d_events = {}
         self._h2d_event_objs = {}  # library-issued copies: the event object each parameter keeps
         self.d2h_events = {}

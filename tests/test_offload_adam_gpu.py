@@ -719,7 +719,7 @@ def test_parameters_without_a_gradient_in_some_passes(fixed_seed, mode, kw):
 
 @pytest.mark.parametrize("mode,clip", [("stochastic_rounding", None), ("fp31_master", 0.05),
                                        ("fp32_master", None)])
-def test_bound_on_pending_write_backs_changes_no_result(fixed_seed, mode, clip, monkeypatch):
+def test_bound_on_pending_write_backs_changes_no_result(fixed_seed, mode, clip):
     """Staging buffers handed back while their write-back still runs are bounded in bytes;
     past the bound the host waits for the oldest write-back.  With a bound of one byte
     (a wait at every issue) and with none, on the hook path and the clipping path: the
@@ -727,15 +727,15 @@ def test_bound_on_pending_write_backs_changes_no_result(fixed_seed, mode, clip, 
     from offload_adam_amd import OffloadAdam
 
     results = []
+    _, default = run_offload_adam(mode, steps=1, ga=1, max_grad_norm=clip)
+    assert default._writeback_pending_limit == max(2 * default._PREFETCH_BYTES, 2 << 30)
     for limit in (1, 1 << 60):
-        monkeypatch.setattr(OffloadAdam, "_WRITEBACK_PENDING_BYTES", limit)
-        model, opt = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip)
+        model, opt = run_offload_adam(mode, steps=3, ga=3, max_grad_norm=clip,
+                                      pending_writeback_bytes=limit)
         assert opt._writeback_pending_limit == limit
         if limit == 1:
             # nothing older than the newest write-back is ever left pending
             assert len(opt._writebacks_pending) <= 1
-        else:
-            assert opt._writeback_pending_bytes > 0  # (the last ones were never waited for)
         torch.cuda.synchronize()
         opt._throttle_writebacks()
         assert opt._writeback_pending_bytes == 0 and not opt._writebacks_pending
