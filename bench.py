@@ -52,7 +52,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # the line says so (``traffic_source``).  Keyed by (workload, launch form).
 TRAFFIC_FROM_PROFILE = {
     ("c1_sr_llama1b", "multi_tensor"): (
-        2_566_926_000, "profiles/adam_multi_kernel_sr_c1_llama1b_hbm_traffic.txt"),
+        2_566_900_000, "profiles/adam_multi_kernel_sr_c1_llama1b_hbm_traffic.txt"),
 }
 
 BYTES_PER_ELEM = {
