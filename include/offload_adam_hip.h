@@ -448,9 +448,8 @@ int oa_link_copy_batch(int count, void* const* dsts, const void* const* srcs,
  * runtime declined, which went through hipMemcpyAsync instead. */
 #define OA_LINK_OFF                 (-10) /* OFFLOAD_ADAM_COPY_ENGINES=off */
 #define OA_LINK_NO_RUNTIME          (-11) /* libhsa-runtime64 or one of its entry points not found */
-#define OA_LINK_NO_STREAM_VALUE_OPS (-12) /* the device offers no signal memory (hipMallocSignalMemory) */
 #define OA_LINK_NO_AGENT            (-13) /* the HIP device was not found among the HSA agents */
-#define OA_LINK_NO_SIGNALS          (-14) /* signal memory could not be obtained or verified */
+#define OA_LINK_NO_SIGNALS          (-14) /* signal memory (hipMallocSignalMemory) could not be obtained or verified */
 int oa_link_copy_status(unsigned* h2d_engine, unsigned* d2h_engine,
                         unsigned long long* h2d_copies, unsigned long long* d2h_copies,
                         unsigned long long* runtime_copies);

@@ -217,11 +217,6 @@ void set_up(DeviceLink& link, int dev) {
   std::call_once(g_hsa_once, load_hsa);
   if (g_switched_off) { link.state = OA_LINK_OFF; return; }
   if (!g_hsa_ok) { link.state = OA_LINK_NO_RUNTIME; return; }
-  int can = 0;
-  if (hipDeviceGetAttribute(&can, hipDeviceAttributeCanUseStreamWaitValue, dev) != hipSuccess || !can) {
-    link.state = OA_LINK_NO_STREAM_VALUE_OPS;
-    return;
-  }
   char busid[64] = {0};
   AgentSearch want{};
   if (hipDeviceGetPCIBusId(busid, sizeof(busid), dev) != hipSuccess ||

@@ -25,8 +25,6 @@ extern "C" const char* oa_error_string(int code) {
       return "offload_adam_hip: fixed-engine copies switched off (OFFLOAD_ADAM_COPY_ENGINES)";
     case OA_LINK_NO_RUNTIME:
       return "offload_adam_hip: the ROCr runtime library or one of its entry points was not found";
-    case OA_LINK_NO_STREAM_VALUE_OPS:
-      return "offload_adam_hip: the device offers no signal memory (hipMallocSignalMemory)";
     case OA_LINK_NO_AGENT:
       return "offload_adam_hip: the HIP device was not found among the HSA agents";
     case OA_LINK_NO_SIGNALS:

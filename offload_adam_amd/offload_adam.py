@@ -88,7 +88,7 @@ def _copy_async(dst, src, kind, stream):
 
     Host<->device copies go through ``oa_h2d_async`` / ``oa_d2h_async``: a fixed SDMA
     engine per direction, chosen inside the library.  Where those are not available
-    (``OFFLOAD_ADAM_COPY_ENGINES=off``, a runtime without stream memory operations)
+    (``OFFLOAD_ADAM_COPY_ENGINES=off``, a runtime that hands out no signal memory)
     the copy is a ``hipMemcpyAsync`` and the HIP runtime picks the engine."""
     nbytes = src.numel() * src.element_size()
     lib = _lib.load()
