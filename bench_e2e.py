@@ -21,6 +21,7 @@ over the host link per step and the achieved H2D / D2H rates against the pinned
 
 import argparse
 import json
+import os
 import math
 import sys
 import time
@@ -792,8 +793,65 @@ def run_resident_adam(args, out, model, loop, torch):
     return out
 
 
+def copy_trace_summary(directory, window_s=None):
+    """Per-direction figures of a ``rocprofv3 --memory-copy-trace --output-format csv``
+    run of this program: copies, busy time (union of the copies' intervals), the sum
+    of their durations (equal to the union when one engine serves the direction) and
+    the time both directions were busy at once - over the last ``window_s`` seconds of
+    the trace (the timed steps: steps x step_s of the run's own output), or all of it.
+    The trace carries time stamps per copy and no byte counts; bytes per step are in
+    this program's output (``h2d_GB_per_step``)."""
+    import csv
+    import glob
+
+    files = glob.glob(os.path.join(directory, "**", "*memory_copy_trace.csv"), recursive=True)
+    if not files:
+        raise SystemExit(f"no *memory_copy_trace.csv under {directory}")
+    per = {}
+    with open(files[0]) as fh:
+        for row in csv.DictReader(fh):
+            per.setdefault(row["Direction"], []).append(
+                (int(row["Start_Timestamp"]), int(row["End_Timestamp"])))
+    end = max(e for v in per.values() for _, e in v)
+    start = end - int(window_s * 1e9) if window_s else min(s for v in per.values() for s, _ in v)
+
+    def merged(intervals):
+        out = []
+        for s, e in sorted(intervals):
+            if out and s <= out[-1][1]:
+                out[-1][1] = max(out[-1][1], e)
+            else:
+                out.append([s, e])
+        return out
+
+    report, unions = {"window_s": round((end - start) / 1e9, 4)}, {}
+    for name, intervals in sorted(per.items()):
+        inside = [(s, e) for s, e in intervals if s >= start]
+        unions[name] = merged(inside)
+        report[name] = {"copies": len(inside),
+                        "busy_s": round(sum(e - s for s, e in unions[name]) / 1e9, 4),
+                        "sum_of_durations_s": round(sum(e - s for s, e in inside) / 1e9, 4)}
+    up = [v for k, v in unions.items() if "HOST_TO_DEVICE" in k]
+    down = [v for k, v in unions.items() if "DEVICE_TO_HOST" in k]
+    if up and down:
+        a, b, i, j, both = up[0], down[0], 0, 0, 0
+        while i < len(a) and j < len(b):
+            both += max(0, min(a[i][1], b[j][1]) - max(a[i][0], b[j][0]))
+            if a[i][1] < b[j][1]:
+                i += 1
+            else:
+                j += 1
+        report["both_directions_busy_s"] = round(both / 1e9, 4)
+    return report
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--copy-trace-summary", metavar="DIR", default=None,
+                    help="no run: summarise the *memory_copy_trace.csv that rocprofv3 "
+                         "--memory-copy-trace wrote under DIR (see --trace-window-s)")
+    ap.add_argument("--trace-window-s", type=float, default=None,
+                    help="with --copy-trace-summary: only the last so many seconds of the trace")
     ap.add_argument("--model", default="llama8b", choices=sorted(MODELS))
     ap.add_argument("--mode", default="stochastic_rounding")
     ap.add_argument("--seq", type=int, default=4096)
@@ -852,6 +910,9 @@ def main():
                          "the HSA tools library when it is loaded.  Default: 'runtime' when the "
                          "tools library is in effect, else 'direct'")
     args = ap.parse_args()
+    if args.copy_trace_summary:
+        print(json.dumps(copy_trace_summary(args.copy_trace_summary, args.trace_window_s)))
+        return
     if args.qat:
         args.mode = "fp32_master"
     if args.runtime_copy_engines:
