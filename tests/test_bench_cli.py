@@ -6,6 +6,8 @@ import subprocess
 import sys
 from pathlib import Path
 
+import pytest
+
 ROOT = Path(__file__).resolve().parents[1]
 sys.path.insert(0, str(ROOT))
 
@@ -107,3 +109,28 @@ def test_summary_is_the_last_key_material_and_stays_small():
     assert "error" in s["steps"]["qat_8b_int4"]
     assert len(json.dumps({"summary": s})) < 1950
     assert bench.summary_of({})["steps"] == {}
+
+
+def test_copy_trace_summary_on_a_synthetic_trace(tmp_path):
+    """bench_e2e.copy_trace_summary: union of intervals per direction, overlap of the two
+    directions, and the trailing window, on a hand-made rocprofv3 memory-copy trace."""
+    import bench_e2e
+
+    rows = [("MEMORY_COPY_HOST_TO_DEVICE", 0, 100), ("MEMORY_COPY_HOST_TO_DEVICE", 50, 150),
+            ("MEMORY_COPY_HOST_TO_DEVICE", 1_000_000_000, 1_400_000_000),
+            ("MEMORY_COPY_DEVICE_TO_HOST", 1_200_000_000, 1_500_000_000),
+            ("MEMORY_COPY_DEVICE_TO_HOST", 1_600_000_000, 2_000_000_000)]
+    sub = tmp_path / "host" / "pid"
+    sub.mkdir(parents=True)
+    with open(sub / "t_memory_copy_trace.csv", "w") as fh:
+        fh.write('"Kind","Direction","Stream_Id","Start_Timestamp","End_Timestamp"\n')
+        for d, s, e in rows:
+            fh.write(f'"MEMORY_COPY","{d}",1,{s},{e}\n')
+    whole = bench_e2e.copy_trace_summary(str(tmp_path))
+    assert whole["MEMORY_COPY_HOST_TO_DEVICE"] == {"copies": 3, "busy_s": 0.4, "sum_of_durations_s": 0.4}
+    assert whole["MEMORY_COPY_DEVICE_TO_HOST"]["busy_s"] == 0.7
+    assert whole["both_directions_busy_s"] == 0.2
+    tail = bench_e2e.copy_trace_summary(str(tmp_path), window_s=1.0)  # from t = 1.0 s on
+    assert tail["MEMORY_COPY_HOST_TO_DEVICE"]["copies"] == 1 and tail["window_s"] == 1.0
+    with pytest.raises(SystemExit):
+        bench_e2e.copy_trace_summary(str(tmp_path / "nothing_here"))
