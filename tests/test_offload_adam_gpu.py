@@ -1588,9 +1588,12 @@ def test_byte_budgets_accept_any_integral_number(value, ok):
         assert build(pinned_limit_bytes=value)._pinned_limit_arg == int(value)
         assert build(prefetch_bytes=np.int64(value))._PREFETCH_BYTES == int(value)
         assert build(grad_cache_bytes=value, state_cache_bytes=np.int32(4096)) is not None
+        assert build(pending_writeback_bytes=value)._writeback_pending_limit == int(value)
     else:
         with pytest.raises(ValueError, match="pinned_limit_bytes"):
             build(pinned_limit_bytes=value)
+        with pytest.raises(ValueError, match="pending_writeback_bytes"):
+            build(pending_writeback_bytes=value)
         if value != "auto":
             with pytest.raises(ValueError, match="prefetch_bytes"):
                 build(prefetch_bytes=value)
